@@ -16,7 +16,8 @@ slots for fixed-size per-request state.
   and tables keep stale contents invisible.
 * **State slots.**  Each live request owns one slot index into per-entry state arenas
   ``[max_requests + 1, *shape]`` (the last slot is scratch for padding rows).  A slot's state is
-  zeroed when it is handed out.  This architecture has no such state; the slots exist anyway.
+  zeroed when it is handed out.  The embedding may keep such state too (``input_state_need``, the arena
+  ``state[INPUT_STATE]``).  A model without any has the slots anyway.
 * **Scratch page.**  Page ``num_blocks`` of every storage is outside the allocator: padding rows
   of fixed-shape decode batches write there (tensorline/paged.py:125-128).
 """
@@ -30,6 +31,8 @@ import torch
 
 from tensorline_amd.cache.allocator import PagePool, page_key
 from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry, StateNeed
+
+INPUT_STATE = "input"      # key of the embedding's state arena beside the schedule entries' (which are keyed by index)
 
 _TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
 
@@ -63,7 +66,8 @@ class _Request:
 class CacheManager:
     def __init__(self, cache_needs: Sequence[CacheNeed | None], schedule: Sequence[ScheduleEntry],
                  state_needs: Sequence[StateNeed | None], *, page_size: int, num_blocks: int, max_requests: int,
-                 dtype: torch.dtype, device, prefix_caching: bool = False, allocate_storage: bool = True):
+                 dtype: torch.dtype, device, prefix_caching: bool = False, allocate_storage: bool = True,
+                 input_state_need: StateNeed | None = None):
         if page_size <= 0 or num_blocks <= 0 or max_requests <= 0:
             raise ValueError("page_size, num_blocks and max_requests must be positive")
         self.page_size, self.num_blocks, self.max_requests = page_size, num_blocks, max_requests
@@ -106,9 +110,10 @@ class CacheManager:
 
         # ---- state slots ----
         self.state_needs = list(state_needs)
-        self.has_state = any(n is not None for n in self.state_needs)
+        self.input_state_need = input_state_need      # what the embedding keeps per request (same slots)
+        self.has_state = any(n is not None for n in self.state_needs) or input_state_need is not None
         self._free_slots: list[int] = list(range(max_requests - 1, -1, -1))
-        self.state: dict[int, torch.Tensor] = {}
+        self.state: dict[int | str, torch.Tensor] = {}
 
         # prefix sharing: only where one page id means the same tokens for every layer and no
         # mixer carries state that pages do not hold
@@ -124,7 +129,7 @@ class CacheManager:
                         plane.name: torch.zeros(plane.storage_shape(num_blocks + 1, page_size),
                                                 dtype=_plane_dtype(plane.dtype, dtype), device=device)
                         for plane in g.need.planes}
-            for i, need in enumerate(self.state_needs):
+            for i, need in list(enumerate(self.state_needs)) + [(INPUT_STATE, input_state_need)]:
                 if need is not None:
                     self.state[i] = torch.zeros((max_requests + 1, *need.shape), dtype=_TORCH_DTYPES[need.dtype], device=device)
 

@@ -216,3 +216,129 @@ extern "C" int tl_gated_scan(const float* gr, const float* gi, int ldg, const fl
     TL_CHECK_LAUNCH("tl_gated_scan");
     return 0;
 }
+
+// ---- convolution, rotation and cache write of an attention layer's projections in one pass ------------------
+// proj float [T, >= C] holds a token's projected queries, keys and values side by side (biases added):
+// Hq query heads of d, Gk key heads of d, Gv value heads of dv; C = (Hq + Gk) d + Gv dv.  Each channel
+// goes through its short causal convolution (taps [C, K], the kept inputs as in tl_causal_conv), then
+//   * queries and keys: the first `rot` dimensions of every head are turned in neighbouring pairs,
+//     (u, v) at dimensions (2i, 2i + 1) -> (u c - v s, v c + u s) with c = mag cos(pos f_i), s = mag
+//     sin(pos f_i), the angle in float (freq null or rot 0: no rotation);
+//   * queries are written to q_out [T, Hq, D] (columns d .. D - 1 are left as they are);
+//   * keys go into k_cache at the token's slot ([pages, page, Gk, D]) and values into v_cache with a
+//     page's tokens innermost ([pages, Gv v_rep, D, page]), every value head v_rep times in a row (a
+//     key head 2g + m then finds the values of g at its own index); padding columns are not written.
+// Gk = 0 (slots null): a layer that only has queries.  A thread per (token, channel); a rotated channel
+// computes its neighbour's convolution as well.  shift != 0 (steps of one token per sequence): the
+// thread also renews what the slot keeps, after every thread of the work-group has read (neighbours
+// lie in one work-group because pairs start at even channels).
+template <typename O>
+__global__ __launch_bounds__(256) void conv_rotate_store_kernel(
+    const float* __restrict__ proj, int ldp, const float* __restrict__ taps, float* __restrict__ kept, long long state_stride,
+    const int32_t* __restrict__ state_slots, const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ pos, const float* __restrict__ freq, float mag, int rot, const int32_t* __restrict__ slots,
+    O* __restrict__ q_out, O* __restrict__ k_cache, O* __restrict__ v_cache, int Hq, int Gk, int d, int Gv, int dv, int D,
+    int v_rep, int page, int C, int K, int shift) {
+    const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    const bool live = c < C;
+    const int s = seq_of_token[t];
+    const int r0 = q_start[s];
+    float* old = kept + (size_t)state_slots[s] * state_stride;
+    const int qk = (Hq + Gk) * d;
+    int head = 0, i = 0;
+    bool turns = false;
+    if (live) {
+        if (c < qk) {
+            head = c / d;
+            i = c - head * d;
+            turns = freq != nullptr && i < rot;
+        } else {
+            head = (c - qk) / dv;
+            i = (c - qk) - head * dv;
+        }
+    }
+    const int c2 = turns ? c - i + (i ^ 1) : c;
+    float mine = 0.f, other = 0.f;
+    float seen[CS_MAX_TAPS];
+    if (live) {
+        for (int j = 0; j < K; ++j) {
+            const int r = t - (K - 1) + j;
+            const float v = r >= r0 ? proj[(size_t)r * ldp + c] : old[(size_t)(r - r0 + K - 1) * C + c];
+            seen[j] = v;
+            mine += taps[(size_t)c * K + j] * v;
+            if (turns) {
+                const float v2 = r >= r0 ? proj[(size_t)r * ldp + c2] : old[(size_t)(r - r0 + K - 1) * C + c2];
+                other += taps[(size_t)c2 * K + j] * v2;
+            }
+        }
+    }
+    if (shift) {
+        __syncthreads();
+        if (live)
+            for (int j = 1; j < K; ++j) old[(size_t)(j - 1) * C + c] = seen[j];
+    }
+    if (!live) return;
+    float y = mine;
+    if (turns) {
+        float sn, cs;
+        sincosf((float)pos[t] * freq[i >> 1], &sn, &cs);
+        sn *= mag;
+        cs *= mag;
+        y = (i & 1) ? mine * cs + other * sn : mine * cs - other * sn;
+    }
+    if (c < Hq * d) {
+        q_out[((size_t)t * Hq + head) * D + i] = tl_from_float<O>(y);
+        return;
+    }
+    const int slot = slots ? slots[t] : -1;
+    if (slot < 0) return;
+    if (c < qk) {
+        k_cache[((size_t)slot * Gk + (head - Hq)) * D + i] = tl_from_float<O>(y);
+        return;
+    }
+    const size_t pg = (size_t)slot / page, within = (size_t)slot % page;
+    for (int r = 0; r < v_rep; ++r)
+        v_cache[((pg * Gv * v_rep + (size_t)head * v_rep + r) * D + i) * page + within] = tl_from_float<O>(y);
+}
+
+// update: 1 renews the kept inputs by a second launch, 2 in the same launch (steps of one token per
+// sequence, T == S; needs rot == 0 or an even d, so that a pair's channels lie in one work-group).
+extern "C" int tl_conv_rotate_store(const float* proj, int ldp, const float* taps, float* kept, long long state_stride,
+                                    const int32_t* state_slots, const int32_t* seq_of_token, const int32_t* q_start,
+                                    const int32_t* pos, const float* freq, float mag, int rot, const int32_t* slots, void* q_out,
+                                    void* k_cache, void* v_cache, int dtype, int T, int S, int Hq, int Gk, int d, int Gv, int dv,
+                                    int D, int v_rep, int page, int K, int update, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && S >= 0 && Hq > 0 && Gk >= 0 && Gv >= 0 && d > 0 && dv > 0 && D >= d && D >= dv && K >= 1 &&
+                     K <= CS_MAX_TAPS && v_rep >= 1,
+                 "tl_conv_rotate_store: bad sizes Hq=%d Gk=%d d=%d Gv=%d dv=%d D=%d taps=%d", Hq, Gk, d, Gv, dv, D, K);
+    const long long C64 = (long long)(Hq + Gk) * d + (long long)Gv * dv;
+    TL_CHECK_ARG(C64 <= (1 << 24) && ldp >= C64 && state_stride >= (long long)(K - 1) * C64,
+                 "tl_conv_rotate_store: rows or the kept inputs are too short");
+    const int C = (int)C64;
+    TL_CHECK_ARG(rot >= 0 && rot % 2 == 0 && rot <= d && (rot == 0 || freq != nullptr), "tl_conv_rotate_store: bad rotation width %d", rot);
+    TL_CHECK_ARG((Gk == 0 && Gv == 0) || (slots && k_cache && v_cache && page > 0 && Gk > 0 && Gv > 0),
+                 "tl_conv_rotate_store: keys and values need their caches and slots");
+    TL_CHECK_ARG(T <= 2147483647 / 2 && tl_ceil_div(C, 256) <= 65535 && S <= 65535, "tl_conv_rotate_store: too large for one launch");
+    TL_CHECK_ARG(update == 1 || (update == 2 && T == S && (rot == 0 || d % 2 == 0)),
+                 "tl_conv_rotate_store: the one-launch form is for steps of one token per sequence");
+    if (T == 0 || S == 0) return 0;
+    if (rot == 0) freq = nullptr;
+    const int shift = update == 2 ? 1 : 0;
+    dim3 block(256), grid(T, tl_ceil_div(C, 256));
+    if (dtype == TL_F32)
+        hipLaunchKernelGGL(conv_rotate_store_kernel<float>, grid, block, 0, stream, proj, ldp, taps, kept, state_stride, state_slots,
+                           seq_of_token, q_start, pos, freq, mag, rot, slots, (float*)q_out, (float*)k_cache, (float*)v_cache, Hq,
+                           Gk, d, Gv, dv, D, v_rep, page, C, K, shift);
+    else if (dtype == TL_BF16)
+        hipLaunchKernelGGL(conv_rotate_store_kernel<bf16_t>, grid, block, 0, stream, proj, ldp, taps, kept, state_stride,
+                           state_slots, seq_of_token, q_start, pos, freq, mag, rot, slots, (bf16_t*)q_out, (bf16_t*)k_cache,
+                           (bf16_t*)v_cache, Hq, Gk, d, Gv, dv, D, v_rep, page, C, K, shift);
+    else return tl_fail("tl_conv_rotate_store: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_conv_rotate_store");
+    if (update == 1 && K > 1) {
+        hipLaunchKernelGGL(causal_conv_keep_kernel, dim3(tl_ceil_div(C, 256), S), block, 0, stream, proj, ldp, kept, state_stride,
+                           state_slots, q_start, C, K);
+        TL_CHECK_LAUNCH("tl_conv_rotate_store keep");
+    }
+    return 0;
+}

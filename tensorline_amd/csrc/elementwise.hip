@@ -56,6 +56,129 @@ extern "C" int tl_embed(const int32_t* ids, const void* table, int table_dtype, 
     return 0;
 }
 
+// ---- embedding gather with a hashed bigram row added ------------------------------------------
+// x[t, :] = float(table[ids[t], :]) + float(bigram[row, :]), row = (prev * mul_prev + ids[t] * mul_cur) mod
+// buckets, where prev is the token ahead of t in its sequence: the row above in the step, or, for the
+// sequence's first row of the step, what its state slot keeps (prev_kept[slot]); a sequence's first token
+// (position 0) reads row `buckets`, the table's last.  The sum is float.
+template <typename T>
+__global__ void embed_bigram_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ pos,
+                                    const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start,
+                                    const int32_t* __restrict__ state_slots, const int32_t* __restrict__ prev_kept,
+                                    long long kept_stride, const T* __restrict__ table, const T* __restrict__ bigram,
+                                    float* __restrict__ x, int H, int V, long long buckets, long long mul_prev,
+                                    long long mul_cur) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* xr = x + (size_t)t * H;
+    if (id < 0 || id >= V) {
+        for (int c = threadIdx.x; c < H; c += blockDim.x) xr[c] = NAN;
+        return;
+    }
+    long long row = buckets;
+    if (pos[t] > 0) {
+        const int s = seq_of_token[t];
+        const long long prev = t > q_start[s] ? ids[t - 1] : prev_kept[(size_t)state_slots[s] * kept_stride];
+        row = (prev * mul_prev + (long long)id * mul_cur) % buckets;
+        if (row < 0) row += buckets;
+    }
+    const T* er = table + (size_t)id * H;
+    const T* br = bigram + (size_t)row * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) xr[c] = tl_to_float(er[c]) + tl_to_float(br[c]);
+}
+
+// A thread per sequence: the slot keeps the sequence's last token of the step.
+__global__ void keep_last_token_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ q_start,
+                                       const int32_t* __restrict__ state_slots, int32_t* __restrict__ prev_kept,
+                                       long long kept_stride, int S) {
+    const int s = blockIdx.x * blockDim.x + threadIdx.x;
+    if (s >= S) return;
+    const int r1 = q_start[s + 1];
+    if (r1 > q_start[s]) prev_kept[(size_t)state_slots[s] * kept_stride] = ids[r1 - 1];
+}
+
+extern "C" int tl_embed_bigram(const int32_t* ids, const int32_t* pos, const int32_t* seq_of_token, const int32_t* q_start,
+                               const int32_t* state_slots, int32_t* prev_kept, long long kept_stride, const void* table,
+                               const void* bigram, int table_dtype, float* x, int T, int S, int H, int V, long long buckets,
+                               long long mul_prev, long long mul_cur, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && S >= 0 && H > 0 && V > 0 && buckets > 0 && kept_stride >= 1, "tl_embed_bigram: bad sizes T=%d H=%d V=%d", T, H, V);
+    if (T == 0 || S == 0) return 0;
+    dim3 grid(T), block(256);
+    if (table_dtype == TL_F32)
+        hipLaunchKernelGGL(embed_bigram_kernel<float>, grid, block, 0, stream, ids, pos, seq_of_token, q_start, state_slots,
+                           prev_kept, kept_stride, (const float*)table, (const float*)bigram, x, H, V, buckets, mul_prev, mul_cur);
+    else if (table_dtype == TL_BF16)
+        hipLaunchKernelGGL(embed_bigram_kernel<bf16_t>, grid, block, 0, stream, ids, pos, seq_of_token, q_start, state_slots,
+                           prev_kept, kept_stride, (const bf16_t*)table, (const bf16_t*)bigram, x, H, V, buckets, mul_prev, mul_cur);
+    else
+        return tl_fail("tl_embed_bigram: unknown dtype %d", table_dtype);
+    TL_CHECK_LAUNCH("tl_embed_bigram");
+    hipLaunchKernelGGL(keep_last_token_kernel, dim3(tl_ceil_div(S, 256)), dim3(256), 0, stream, ids, q_start, state_slots,
+                       prev_kept, kept_stride, S);
+    TL_CHECK_LAUNCH("tl_embed_bigram keep");
+    return 0;
+}
+
+// ---- a normed branch added to the stream, and the next norm -------------------------------------
+// A residual branch whose output y is RMS-normed before it joins the stream:
+//   x[r] += mult * y[r] / sqrt(mean(y[r]^2) + eps_b) * wb
+// and, with w, the norm that reads the stream next, out[r] = x[r] / sqrt(mean(x[r]^2) + eps) * w, in the
+// same pass.  With `rows`: out only, for x[rows[r]] and y[rows[r]]; x is left as it is.  Float sums.
+template <typename O, bool HAS_ROWS>
+__global__ __launch_bounds__(1024) void branch_norm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                               const float* __restrict__ wb, float mult, float eps_b,
+                                                               const float* __restrict__ w, float eps, O* __restrict__ out,
+                                                               const int32_t* __restrict__ rows, int H) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t src = HAS_ROWS ? (size_t)rows[r] : (size_t)r;
+    float* xr = x + src * H;
+    const float* yr = y + src * H;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) ss += yr[c] * yr[c];
+    ss = tl_block_sum(ss, red);
+    const float f = mult / sqrtf(ss / (float)H + eps_b);
+    float sx = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        const float v = xr[c] + yr[c] * f * wb[c];
+        if (!HAS_ROWS) xr[c] = v;
+        sx += v * v;
+    }
+    if (!w) return;
+    sx = tl_block_sum(sx, red);
+    const float rstd = 1.0f / sqrtf(sx / (float)H + eps);
+    O* orow = out + (size_t)r * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        const float v = HAS_ROWS ? xr[c] + yr[c] * f * wb[c] : xr[c];
+        orow[c] = tl_from_float<O>(v * rstd * w[c]);
+    }
+}
+
+extern "C" int tl_branch_norm_add(float* x, const float* y, const float* wb, float mult, float eps_b, const float* w, float eps,
+                                  void* out, int out_dtype, const int32_t* rows, int n_rows, int H, hipStream_t stream) {
+    TL_CHECK_ARG(n_rows >= 0 && H > 0 && eps >= 0.f && eps_b >= 0.f, "tl_branch_norm_add: bad sizes rows=%d H=%d", n_rows, H);
+    TL_CHECK_ARG((w == nullptr) == (out == nullptr) && (rows == nullptr || w != nullptr), "tl_branch_norm_add: a norm needs its output, and rows a norm");
+    if (n_rows == 0) return 0;
+    int threads = ((H + 63) / 64) * 64;
+    if (threads > 1024) threads = 1024;
+    dim3 grid(n_rows), block(threads);
+#define TL_BRANCH_CASE(OT)                                                                                                       \
+    do {                                                                                                                         \
+        if (rows)                                                                                                                \
+            hipLaunchKernelGGL((branch_norm_add_kernel<OT, true>), grid, block, 0, stream, x, y, wb, mult, eps_b, w, eps, (OT*)out, \
+                               rows, H);                                                                                         \
+        else                                                                                                                     \
+            hipLaunchKernelGGL((branch_norm_add_kernel<OT, false>), grid, block, 0, stream, x, y, wb, mult, eps_b, w, eps,          \
+                               (OT*)out, rows, H);                                                                               \
+    } while (0)
+    if (out_dtype == TL_BF16) TL_BRANCH_CASE(bf16_t);
+    else if (out_dtype == TL_F32) TL_BRANCH_CASE(float);
+    else return tl_fail("tl_branch_norm_add: unknown dtype %d", out_dtype);
+#undef TL_BRANCH_CASE
+    TL_CHECK_LAUNCH("tl_branch_norm_add");
+    return 0;
+}
+
 // ---- residual add + RMSNorm ----------------------------------------------------------------
 // Without `rows`: x[r] += residual[r] (written back, float), out[r] = x[r] * rstd * w.
 // With `rows`:    out[r] = norm(x[rows[r]] + residual[rows[r]]); x is left as it is.

@@ -2,13 +2,14 @@
 // the experts' products as one grouped launch each, and the weighted sum per token.
 //
 //   tl_moe_route    per token: the `top` largest router logits (lowest index wins a tie) and their weights:
-//                   the softmax over those alone, or scale * sigmoid of each  -> expert ids, weights [T, top]
+//                   the softmax over those alone, scale * sigmoid of each, or their shares of the softmax
+//                   over all experts                             -> expert ids, weights [T, top]
 //   tl_moe_sort     the (token, choice) pairs ordered by expert and cut into row tiles of BM rows that
 //                   hold one expert's pairs only                 -> order, tiles
 //   tl_moe_gemm     a product per tile with its expert's matrix: gate/up with the gated activation
 //                   min(g, limit) sigmoid(alpha min(g, limit)) (clamp(u, +-limit) + shift) in the epilogue
-//                   (limit = infinity, alpha = 1, shift = 0: silu(g) u), or down, which scatters rows back
-//                   to their pairs
+//                   (limit = infinity, alpha = 1, shift = 0: silu(g) u), or up alone with the square of relu
+//                   in the epilogue (experts without gate), or down, which scatters rows back to their pairs
 //   tl_moe_combine  out[t] = sum over the token's choices, in the order of its choices, of weight *
 //                   row (+ a shared expert's output)
 //
@@ -73,19 +74,27 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
     const float largest = __shfl(my_val, 0, 64);
     const float ex = lane < top ? expf(my_val - largest) : 0.f;
-    const float sum = tl_wave_sum(ex);
+    float sum;
+    if (mode == 2) {                    // the softmax over all experts, the chosen ones' shares kept as they are
+        float all = 0.f;
+        for (int e = lane; e < E; e += 64) all += expf(z[e] - largest);
+        sum = tl_wave_sum(all);
+    } else {
+        sum = tl_wave_sum(ex);
+    }
     if (lane < top) {
         ids[(size_t)t * top + lane] = my_id;
         weights[(size_t)t * top + lane] = ex / sum;
     }
 }
 
-// mode 0: weights = softmax over the chosen logits; mode 1: weights = scale * sigmoid(chosen logit).
+// mode 0: weights = softmax over the chosen logits; mode 1: weights = scale * sigmoid(chosen logit);
+// mode 2: weights = the chosen experts' shares of the softmax over all logits, not renormalised.
 extern "C" int tl_moe_route(const float* logits, int ldl, int32_t* ids, float* weights, int T, int E, int top, int mode,
                             float scale, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && E > 0 && top > 0 && top <= E && top <= MOE_MAX_TOP && E <= MOE_MAX_EXPERTS && ldl >= E,
                  "tl_moe_route: bad sizes E=%d top=%d", E, top);
-    TL_CHECK_ARG(mode == 0 || mode == 1, "tl_moe_route: unknown weighting %d", mode);
+    TL_CHECK_ARG(mode >= 0 && mode <= 2, "tl_moe_route: unknown weighting %d", mode);
     if (T == 0) return 0;
     hipLaunchKernelGGL(moe_route_kernel, dim3(tl_ceil_div(T, 4)), dim3(256), 0, stream, logits, ldl, ids, weights, T, E, top, mode, scale);
     TL_CHECK_LAUNCH("tl_moe_route");
@@ -178,11 +187,14 @@ template <> __device__ __forceinline__ float4 mg_load4<bf16_t>(const bf16_t* __r
 // (order[place] / top), C [P, N] by place, C = act(gate, up).  Otherwise: W [E, N, K], A [P, K] by
 // place, C [P, N] by pair (order[place]).  Four waves side by side, each MB x NB blocks of 16 x 16
 // (GLU: NB gate blocks and NB up blocks).
-template <typename TA, typename TW, typename TO, int MB, int NB, bool GLU>
+// MODE 0: down; 1: gate and up with the gated activation; 2: up alone, A rows gathered by token and C by
+// place as for 1, W [E, N, K], C = max(., 0)^2.
+template <typename TA, typename TW, typename TO, int MB, int NB, int MODE>
 __global__ __launch_bounds__(MG_THREADS) void moe_gemm_kernel(const TA* __restrict__ A, int lda, const TW* __restrict__ W,
                                                              TO* __restrict__ C, int ldc, const int32_t* __restrict__ order,
                                                              const int32_t* __restrict__ tiles, int top, int N, int K,
                                                              int a_vec, int w_vec, float limit, float alpha, float shift) {
+    constexpr bool GLU = MODE == 1, BY_TOKEN = MODE != 0;
     constexpr int BM = MB * 16, BN = 4 * NB * 16, WR = GLU ? 2 * BN : BN, NW = GLU ? 2 * NB : NB;
     constexpr int A_PIECES = BM * 4, W_PIECES = WR * 4;
     constexpr int A_PER = (A_PIECES + MG_THREADS - 1) / MG_THREADS, W_PER = (W_PIECES + MG_THREADS - 1) / MG_THREADS;
@@ -194,7 +206,7 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_kernel(const TA* __restri
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, lg = lane >> 4;
     const int n0 = blockIdx.x * BN;
-    for (int r = tid; r < BM; r += MG_THREADS) arow[r] = r < rows ? (GLU ? order[place0 + r] / top : place0 + r) : -1;
+    for (int r = tid; r < BM; r += MG_THREADS) arow[r] = r < rows ? (BY_TOKEN ? order[place0 + r] / top : place0 + r) : -1;
     __syncthreads();
     const TW* We = W + (size_t)e * (GLU ? 2 : 1) * N * K;
 
@@ -282,6 +294,9 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_kernel(const TA* __restri
                     const float g = fminf(acc[i][j][v], limit);
                     const float u = fminf(fmaxf(acc[i][NB + j][v], -limit), limit);
                     C[(size_t)(place0 + r) * ldc + n] = tl_from_float<TO>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + shift));
+                } else if (MODE == 2) {
+                    const float u = fmaxf(acc[i][j][v], 0.f);
+                    C[(size_t)(place0 + r) * ldc + n] = tl_from_float<TO>(u * u);
                 } else {
                     C[(size_t)order[place0 + r] * ldc + n] = tl_from_float<TO>(acc[i][j][v]);
                 }
@@ -299,12 +314,13 @@ typedef __bf16 mg_bf16x8 __attribute__((ext_vector_type(8)));
 #define MGB_KT 64
 #define MGB_LD 72
 
-template <int MB, bool GLU>
+template <int MB, int MODE>
 __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda,
                                                                   const bf16_t* __restrict__ W, void* __restrict__ Cv, int ldc,
                                                                   const int32_t* __restrict__ order,
                                                                   const int32_t* __restrict__ tiles, int top, int N, int K,
                                                                   float limit, float alpha, float shift) {
+    constexpr bool GLU = MODE == 1, BY_TOKEN = MODE != 0;
     constexpr int BM = MB * 16, WR = 128, BN = GLU ? 64 : 128;
     constexpr int A_PIECES = BM * 8, W_PIECES = WR * 8;
     constexpr int A_PER = (A_PIECES + MG_THREADS - 1) / MG_THREADS, W_PER = W_PIECES / MG_THREADS;
@@ -316,7 +332,7 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * BN;
-    for (int r = tid; r < BM; r += MG_THREADS) arow[r] = r < rows ? (GLU ? order[place0 + r] / top : place0 + r) : -1;
+    for (int r = tid; r < BM; r += MG_THREADS) arow[r] = r < rows ? (BY_TOKEN ? order[place0 + r] / top : place0 + r) : -1;
     __syncthreads();
     const bf16_t* We = W + (size_t)e * (GLU ? 2 : 1) * N * K;
 
@@ -407,6 +423,14 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
                 const float up = fminf(fmaxf(acc[i][1][v], -limit), limit);
                 reinterpret_cast<bf16_t*>(Cv)[(size_t)(place0 + r) * ldc + n] =
                     tl_from_float<bf16_t>(gt * (1.0f / (1.0f + expf(-alpha * gt))) * (up + shift));
+            } else if (MODE == 2) {
+                bf16_t* crow = reinterpret_cast<bf16_t*>(Cv) + (size_t)(place0 + r) * ldc;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int n = n0 + wave * 32 + j * 16 + c;
+                    const float u = fmaxf(acc[i][j][v], 0.f);
+                    if (n < N) crow[n] = tl_from_float<bf16_t>(u * u);
+                }
             } else {
                 float* crow = reinterpret_cast<float*>(Cv) + (size_t)order[place0 + r] * ldc;
 #pragma unroll
@@ -419,6 +443,7 @@ __global__ __launch_bounds__(MG_THREADS) void moe_gemm_bf16_kernel(const bf16_t*
 }
 
 // glu 1: A [T, K] tokens (row stride lda), W [E, 2N, K], C [P, N] by place, of type c_dtype.
+// glu 2: the same without gate: W [E, N, K], C = max(A W^T, 0)^2.
 // glu 0: A [P, K] by place, W [E, N, K], C float [P, N] by pair.  max_tiles bounds the tiles that
 // tl_moe_sort can have made: P / BM + E.
 extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, int w_dtype, void* C, int c_dtype, int ldc,
@@ -426,6 +451,7 @@ extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, i
                            float limit, float alpha, float shift, hipStream_t stream) {
     TL_CHECK_ARG(N > 0 && K > 0 && lda >= K && ldc >= N && top > 0 && (BM == 16 || BM == 64), "tl_moe_gemm: bad sizes N=%d K=%d BM=%d", N, K, BM);
     TL_CHECK_ARG(max_tiles >= 0 && max_tiles <= 65535, "tl_moe_gemm: %d row tiles are too many for one launch", max_tiles);
+    TL_CHECK_ARG(glu >= 0 && glu <= 2, "tl_moe_gemm: unknown form %d", glu);
     if (max_tiles == 0) return 0;
     const size_t a_el = a_dtype == TL_F32 ? 4 : 2, w_el = w_dtype == TL_F32 ? 4 : 2;
     const int a_vec = ((uintptr_t)A % (4 * a_el) == 0 && lda % 4 == 0) ? 1 : 0;
@@ -442,26 +468,33 @@ extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, i
     const bool bf = a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == (glu ? TL_BF16 : TL_F32);
     if (bf && K % 8 == 0 && lda % 8 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0) {
 #define GO_BF(MB, GLU)                                                                                                   \
-    hipLaunchKernelGGL((moe_gemm_bf16_kernel<MB, GLU>), dim3(tl_ceil_div(N, GLU ? 64 : 128), max_tiles), dim3(MG_THREADS), 0, \
+    hipLaunchKernelGGL((moe_gemm_bf16_kernel<MB, GLU>), dim3(tl_ceil_div(N, GLU == 1 ? 64 : 128), max_tiles), dim3(MG_THREADS), 0, \
                        stream, (const bf16_t*)A, lda, (const bf16_t*)W, C, ldc, order, tiles, top, N, K, limit, alpha, shift)
-        if (glu) {
-            if (BM == 16) GO_BF(1, true);
-            else GO_BF(4, true);
+        if (glu == 1) {
+            if (BM == 16) GO_BF(1, 1);
+            else GO_BF(4, 1);
+        } else if (glu == 2) {
+            if (BM == 16) GO_BF(1, 2);
+            else GO_BF(4, 2);
         } else {
-            if (BM == 16) GO_BF(1, false);
-            else GO_BF(4, false);
+            if (BM == 16) GO_BF(1, 0);
+            else GO_BF(4, 0);
         }
 #undef GO_BF
         TL_CHECK_LAUNCH("tl_moe_gemm");
         return 0;
     }
-    if (glu) {
-        if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32) GO_BM(float, float, float, true);
-        else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_BF16) GO_BM(bf16_t, bf16_t, bf16_t, true);
+    if (glu == 1) {
+        if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32) GO_BM(float, float, float, 1);
+        else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_BF16) GO_BM(bf16_t, bf16_t, bf16_t, 1);
+        else return tl_fail("tl_moe_gemm: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
+    } else if (glu == 2) {
+        if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32) GO_BM(float, float, float, 2);
+        else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_BF16) GO_BM(bf16_t, bf16_t, bf16_t, 2);
         else return tl_fail("tl_moe_gemm: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
     } else {
-        if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32) GO_BM(float, float, float, false);
-        else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_F32) GO_BM(bf16_t, bf16_t, float, false);
+        if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32) GO_BM(float, float, float, 0);
+        else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_F32) GO_BM(bf16_t, bf16_t, float, 0);
         else return tl_fail("tl_moe_gemm: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
     }
 #undef GO_BM

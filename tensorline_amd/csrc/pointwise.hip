@@ -556,3 +556,49 @@ extern "C" int tl_scaled_sum(const float* x, const float* y, float* out, float a
     TL_CHECK_LAUNCH("tl_scaled_sum");
     return 0;
 }
+
+// ---- the difference of two attention maps, normed per head ---------------------------------------------------
+// a [T, 2 H, D]: what attention leaves for 2 H query heads that are the two maps of H heads, ordered by
+// key/value head g, then map m, then the head's place r within its group of R = H / G:
+// head (2 g + m) R + r is map m of head g R + r; the first dv of its D columns count.
+// out [T, H, dv]: o = a1 - lambda a2, divided by its root mean square over the dv values (eps inside
+// the root), times `post`.  A wave per (token, head); float arithmetic.
+template <typename T>
+__global__ __launch_bounds__(256) void diff_combine_kernel(const T* __restrict__ a, int lda, T* __restrict__ out, int n, int H,
+                                                          int G, int dv, int D, float lambda, float eps, float post) {
+    const int lane = threadIdx.x & 63;
+    const int item = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (item >= n) return;
+    const int t = item / H, h = item - t * H;
+    const int R = H / G, g = h / R, r = h - g * R;
+    const T* a1 = a + (size_t)t * lda + (size_t)((2 * g) * R + r) * D;
+    const T* a2 = a + (size_t)t * lda + (size_t)((2 * g + 1) * R + r) * D;
+    float ss = 0.f;
+    for (int c = lane; c < dv; c += 64) {
+        const float o = tl_to_float(a1[c]) - lambda * tl_to_float(a2[c]);
+        ss += o * o;
+    }
+    ss = tl_wave_sum(ss);
+    const float f = post / sqrtf(ss / (float)dv + eps);
+    T* orow = out + ((size_t)t * H + h) * dv;
+    for (int c = lane; c < dv; c += 64) orow[c] = tl_from_float<T>((tl_to_float(a1[c]) - lambda * tl_to_float(a2[c])) * f);
+}
+
+extern "C" int tl_diff_combine(const void* a, int lda, void* out, int dtype, int T, int H, int G, int dv, int D, float lambda,
+                               float eps, float post, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && H > 0 && G > 0 && H % G == 0 && dv > 0 && D >= dv && lda >= 2 * H * D && eps >= 0.f,
+                 "tl_diff_combine: bad sizes H=%d G=%d dv=%d D=%d", H, G, dv, D);
+    TL_CHECK_ARG((long long)T * H <= 2147483647LL, "tl_diff_combine: too many rows");
+    if (T == 0) return 0;
+    const int n = T * H;
+    dim3 grid(tl_ceil_div(n, 4)), block(256);
+    if (dtype == TL_F32)
+        hipLaunchKernelGGL(diff_combine_kernel<float>, grid, block, 0, stream, (const float*)a, lda, (float*)out, n, H, G, dv, D,
+                           lambda, eps, post);
+    else if (dtype == TL_BF16)
+        hipLaunchKernelGGL(diff_combine_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)a, lda, (bf16_t*)out, n, H, G, dv, D,
+                           lambda, eps, post);
+    else return tl_fail("tl_diff_combine: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_diff_combine");
+    return 0;
+}

@@ -71,6 +71,7 @@ class StepContext:
     host_ctx_start: list[int] = field(default_factory=list)
     host_state_slots: list[int] = field(default_factory=list)
     logits_for_all_rows: bool = False  # logit_rows is 0, 1, .., T-1: no gather is needed
+    input_state: torch.Tensor | None = None   # [slots + 1, *shape]: what the embedding keeps per request, if anything
 
 
 @dataclass

@@ -49,7 +49,8 @@ class TraceSession:
         self.model = model
         self.cache = CacheManager(model.cache_needs(), model.schedule, model.state_needs(), page_size=page_size,
                                   num_blocks=num_blocks, max_requests=max_requests, dtype=model.dtype,
-                                  device=model.device, prefix_caching=False)
+                                  device=model.device, prefix_caching=False,
+                                  input_state_need=model.input_state_need())
         if graphs:
             from tensorline_amd.engine.graphs import GraphRunner
             # one request can hold the whole pool at most: that bounds every page table

@@ -14,7 +14,7 @@ from typing import Sequence
 import numpy as np
 import torch
 
-from tensorline_amd.cache.manager import CacheManager
+from tensorline_amd.cache.manager import INPUT_STATE, CacheManager
 from tensorline_amd.engine.batch import LayerCache, PackedBatch, StepContext, StepEntry, pack_batch
 from tensorline_amd.models.decoder import DecoderModel
 
@@ -80,7 +80,8 @@ class ModelRunner:
             state_slots=view("state_slots"), logit_rows=view("logit_rows"), facts=packed.facts,
             host_q_start=packed.host_q_start, host_ctx_start=packed.host_ctx_start,
             host_state_slots=packed.host_state_slots, logits_for_all_rows=packed.logits_for_all_rows,
-            extra={name[6:]: view(name) for name in packed.offsets if name.startswith("extra:")})
+            extra={name[6:]: view(name) for name in packed.offsets if name.startswith("extra:")},
+            input_state=self.cache.state.get(INPUT_STATE))
         cache = self.cache
         g_slots = [view(f"slots{g}") for g in range(len(cache.groups))]
         g_tables = [view(f"tables{g}").view(packed.S, packed.group_nb[g]) for g in range(len(cache.groups))]

@@ -103,6 +103,11 @@ class DecoderModel:
         """Per schedule entry: the fixed-size per-request state its block keeps, or None."""
         return [self.blocks[e.layer].state_need() for e in self.schedule]
 
+    def input_state_need(self) -> StateNeed | None:
+        """The fixed-size per-request state the embedding keeps (the token before, say), or None."""
+        fn = getattr(self.embedding, "state_need", None)
+        return fn() if fn is not None else None
+
     # ---- one step ------------------------------------------------------------------------
     def tune_library(self, rows: int) -> int:
         """Let the library choose its kernels by measurement for steps of ``rows`` tokens (a full
@@ -123,7 +128,8 @@ class DecoderModel:
         if getattr(self.head, "takes_normed_rows", lambda: False)():
             fn = getattr(self.final_norm, "deferrable", None)
             carried = fn() if fn is not None else None
-        return Intake(carried, bool(getattr(self.final_norm, "adds_share_sums", False)))
+        return Intake(carried, bool(getattr(self.final_norm, "adds_share_sums", False)),
+                      bool(getattr(self.final_norm, "adds_normed_branch", False)))
 
     def _negotiate(self) -> list[Intake | None]:
         """For every schedule entry the intake of whoever runs after it, or None for a block that
@@ -155,7 +161,8 @@ class DecoderModel:
         """``caches[i]`` is the view of the cache for schedule entry ``i``."""
         if self._after is None:
             self._after = self._negotiate()
-        x = self.embedding.forward(ctx.ids)
+        step = getattr(self.embedding, "forward_step", None)     # an embedding that looks at more than the ids
+        x = step(ctx) if step is not None else self.embedding.forward(ctx.ids)
         again = x.clone() if any(e.add_input for e in self.schedule) else None   # the stream is updated in place
         carry = None
         for i, e in enumerate(self.schedule):

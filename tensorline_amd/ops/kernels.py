@@ -119,12 +119,74 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = Non
     return out
 
 
+def embed_bigram(ids: torch.Tensor, ctx, table: torch.Tensor, bigram: torch.Tensor, kept: torch.Tensor, mul_prev: int,
+                 mul_cur: int) -> torch.Tensor:
+    """``x[t] = float(table[ids[t]]) + float(bigram[row_t])`` in float32, ``row_t = (prev_t * mul_prev + ids[t] * mul_cur)
+    mod buckets`` with ``prev_t`` the token ahead of t in its sequence and ``buckets = bigram.shape[0] - 1``; a sequence's
+    first token (position 0) reads the last row.  ``kept`` int32 [slots, >= 1]: column 0 of a request's slot holds its last
+    token; it is read for a sequence's first row of the step and renewed afterwards."""
+    _on_gpu(ids, table, bigram, kept)
+    _i32(ids, "ids")
+    T, (V, H) = ids.numel(), table.shape
+    _check(table.dim() == 2 and table.is_contiguous() and bigram.dim() == 2 and bigram.is_contiguous()
+           and bigram.shape[1] == H and bigram.shape[0] >= 2 and bigram.dtype == table.dtype,
+           "embed_bigram: the tables must be contiguous [V, H] and [buckets + 1, H] of one dtype")
+    _check(kept.dtype == torch.int32 and kept.dim() == 2 and kept.stride(1) == 1, "embed_bigram: the kept tokens must be int32 [slots, n]")
+    _i32(ctx.pos, "pos", T)
+    _i32(ctx.seq_of_token, "seq_of_token", T)
+    out = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    _call("tl_embed_bigram", _ptr(ids), _ptr(ctx.pos), _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(ctx.state_slots),
+          _ptr(kept), ctypes.c_longlong(kept.stride(0)), _ptr(table), _ptr(bigram), _code(table, "embed_bigram"), _ptr(out), T,
+          ctx.num_seqs, H, V, ctypes.c_longlong(bigram.shape[0] - 1), ctypes.c_longlong(int(mul_prev)),
+          ctypes.c_longlong(int(mul_cur)), _stream())
+    return out
+
+
+@dataclass
+class NormedBranch:
+    """The output of a residual branch that is RMS-normed before it joins the stream: stands for
+    ``mult * rms_norm(y, weight, eps)``, still to be added.  The norm that reads the stream next adds it in
+    its own pass (:func:`add_rmsnorm`)."""
+    y: torch.Tensor          # float32 [T, H]
+    weight: torch.Tensor     # float32 [H]
+    eps: float
+    mult: float
+
+
+def add_normed_branch(x: torch.Tensor, branch: NormedBranch) -> None:
+    """``x += branch.mult * rms_norm(branch.y) * branch.weight`` in place, nothing else."""
+    _branch_norm_add(x, branch, None, 0.0, None, None)
+
+
+def _branch_norm_add(x, branch: NormedBranch, weight, eps, out_dtype, rows):
+    y, wb = branch.y, branch.weight
+    _on_gpu(x, y, wb, weight, rows)
+    _check(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "normed branch: x must be contiguous float32 [T, H]")
+    T, H = x.shape
+    _check(y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (T, H), "normed branch: the branch must be float32 and match x")
+    _f32(wb, "normed branch weight", H)
+    out, n = None, T
+    if weight is not None:
+        _f32(weight, "norm weight", H)
+        if rows is not None:
+            _i32(rows, "rows")
+            n = rows.numel()
+        out = torch.empty(n, H, dtype=out_dtype, device=x.device)
+    _call("tl_branch_norm_add", _ptr(x), _ptr(y), _ptr(wb), ctypes.c_float(branch.mult), ctypes.c_float(branch.eps), _ptr(weight),
+          ctypes.c_float(eps), _ptr(out), _code(out, "normed branch out") if out is not None else F32, _ptr(rows), n, H, _stream())
+    return out
+
+
 def add_rmsnorm(x: torch.Tensor, residual: "torch.Tensor | ShareSum | None", weight: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: torch.Tensor | None = None,
                 out: torch.Tensor | None = None) -> torch.Tensor:
     """Without ``rows``: ``x += residual`` in place (float32), returns ``RMSNorm(x) * weight``.
     With ``rows``: returns the norm of ``x[rows] + residual[rows]`` and leaves ``x`` alone.
-    ``residual`` may be a :class:`ShareSum`: its shares are added in order, then to ``x``."""
+    ``residual`` may be a :class:`ShareSum`: its shares are added in order, then to ``x``; or a
+    :class:`NormedBranch`: it is normed first, scaled and added."""
+    if isinstance(residual, NormedBranch):
+        _check(out is None, "add_rmsnorm: a normed branch comes with an output of its own")
+        return _branch_norm_add(x, residual, weight, eps, out_dtype, rows)
     parts, part_stride = 1, 0
     if isinstance(residual, ShareSum):
         residual = residual.parts
@@ -1222,18 +1284,22 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ctx, st
 
 # ---------------------------------------------------------------------------------------------
 # Routed experts
+ROUTER_WEIGHTINGS = {"softmax_top": 0, "sigmoid": 1, "softmax_all": 2}
+
+
 def moe_route(logits: torch.Tensor, top: int, weighting: str = "softmax_top", scale: float = 1.0) -> tuple[torch.Tensor, torch.Tensor]:
     """Per row of float32 ``logits`` [T, E]: the ``top`` largest (lowest index first among equals), as
     int32 ids [T, top], and their weights, float32 [T, top]: the softmax over those alone
-    (``weighting`` "softmax_top"), or ``scale * sigmoid(logit)`` of each, not renormalised ("sigmoid")."""
-    _check(weighting in ("softmax_top", "sigmoid"), f"moe_route: unknown weighting {weighting!r}")
+    (``weighting`` "softmax_top"), ``scale * sigmoid(logit)`` of each, not renormalised ("sigmoid"), or their
+    shares of the softmax over all E logits, not renormalised ("softmax_all")."""
+    _check(weighting in ROUTER_WEIGHTINGS, f"moe_route: unknown weighting {weighting!r}")
     _on_gpu(logits)
     T, E = logits.shape
     _check(logits.dtype == torch.float32 and logits.stride(1) == 1, "moe_route: logits must be float32 [T, E]")
     ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     weights = torch.empty(T, top, dtype=torch.float32, device=logits.device)
     _call("tl_moe_route", _ptr(logits), logits.stride(0) if T > 1 else E, _ptr(ids), _ptr(weights), T, E, int(top),
-          1 if weighting == "sigmoid" else 0, ctypes.c_float(scale), _stream())
+          ROUTER_WEIGHTINGS[weighting], ctypes.c_float(scale), _stream())
     return ids, weights
 
 
@@ -1243,16 +1309,18 @@ def moe_tile_rows(pairs: int, experts: int) -> int:
 
 
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
-                limit: float, alpha: float, shared: torch.Tensor | None = None, shift: float = 1.0) -> torch.Tensor:
+                limit: float, alpha: float, shared: torch.Tensor | None = None, shift: float = 1.0,
+                gated: bool = True) -> torch.Tensor:
     """``out[t] = sum_c weights[t, c] * expert_{ids[t, c]}(h[t]) (+ shared[t])`` in float32, where expert
     e is ``down[e] @ act(gate_up[e] @ h)`` with the gated activation ``g' sigmoid(alpha g') (u' + shift)``,
     ``g' = min(g, limit)``, ``u' = clamp(u, -limit, limit)`` (:func:`clamp_glu` has ``shift`` 1; an infinite
     ``limit`` with ``alpha`` 1 and ``shift`` 0 is ``silu(g) * u``).
-    ``gate_up`` [E, 2F, K] (gate rows first), ``down`` [E, N, F]; ``h`` [T, K] in the weights' dtype."""
+    ``gate_up`` [E, 2F, K] (gate rows first), ``down`` [E, N, F]; ``h`` [T, K] in the weights' dtype.
+    ``gated`` False: experts without gate, ``down[e] @ relu(up[e] @ h)^2`` with ``gate_up`` = up [E, F, K]."""
     _on_gpu(h, gate_up, down, ids, weights, shared)
     T, K = h.shape
     E, F2, _ = gate_up.shape
-    F, N, top = F2 // 2, down.shape[1], ids.shape[1]
+    F, N, top = (F2 // 2 if gated else F2), down.shape[1], ids.shape[1]
     _check(h.stride(1) == 1 and gate_up.is_contiguous() and down.is_contiguous() and gate_up.shape[2] == K
            and tuple(down.shape) == (E, N, F) and h.dtype == gate_up.dtype == down.dtype, "moe_experts: bad shapes")
     _check(ids.dtype == torch.int32 and ids.is_contiguous() and tuple(ids.shape) == (T, top), "moe_experts: bad ids")
@@ -1268,7 +1336,7 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids:
     act = torch.empty(P, F, dtype=h.dtype, device=h.device)
     _call("tl_moe_gemm", _ptr(h), _code(h, "moe_experts input"), h.stride(0) if T > 1 else K, _ptr(gate_up),
           _code(gate_up, "moe_experts weights"), _ptr(act), _code(act, "moe_experts"), F, _ptr(order), _ptr(tiles), max_tiles, BM,
-          top, F, K, 1, ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift), _stream())
+          top, F, K, 1 if gated else 2, ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(shift), _stream())
     y = torch.empty(P, N, dtype=torch.float32, device=h.device)
     _call("tl_moe_gemm", _ptr(act), _code(act, "moe_experts"), F, _ptr(down), _code(down, "moe_experts weights"), _ptr(y), F32, N,
           _ptr(order), _ptr(tiles), max_tiles, BM, top, N, F, 0, ctypes.c_float(0.0), ctypes.c_float(0.0), ctypes.c_float(0.0),
@@ -1368,3 +1436,68 @@ def qk_norm_store(proj: torch.Tensor, pos: torch.Tensor, q_weight: torch.Tensor 
           ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every), _ptr(slots), _ptr(q), _ptr(k_cache), _ptr(v_cache),
           _code(q, "qk_norm_store"), T, heads, kv_heads, dim, vdim, D, page, _stream())
     return q
+
+
+def conv_rotate_store(proj: torch.Tensor, taps: torch.Tensor, ctx, state: torch.Tensor, offset: int, freq: torch.Tensor | None,
+                      mag: float, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, slots: torch.Tensor | None,
+                      heads: int, k_heads: int, dim: int, v_heads: int, vdim: int, head_size: int, v_repeat: int,
+                      out_dtype: torch.dtype) -> torch.Tensor:
+    """What lies between the fused q/k/v projection of an attention layer with short convolutions and attention, in
+    one pass per token.  ``proj`` float32 [T, >= C], C = (heads + k_heads) * dim + v_heads * vdim, biases added
+    (columns beyond C are not looked at).  Every channel goes through its causal convolution (``taps`` float32 [C, K];
+    the inputs ahead of the step's first row are the K - 1 rows kept at ``state[slot, offset : offset + (K - 1) C]``,
+    renewed afterwards); queries and keys are then turned in neighbouring pairs (2i, 2i + 1) over their first
+    ``2 * len(freq)`` dimensions by the angle ``pos * freq[i]``, cosine and sine times ``mag`` (``freq`` None: no
+    rotation); keys and values go into the cache pages at ``slots`` (``k_cache`` [pages, page, k_heads, head_size],
+    ``v_cache`` [pages, v_heads * v_repeat, head_size, page], every value head ``v_repeat`` times in a row).  ``k_heads``
+    0: a layer that only has queries (no caches).  Returns the queries [T, heads * head_size] in ``out_dtype``, zeros
+    beyond ``dim`` in every head."""
+    _on_gpu(proj, taps, state, freq, k_cache, v_cache, slots)
+    T = proj.shape[0]
+    C = (heads + k_heads) * dim + v_heads * vdim
+    K = taps.shape[1]
+    _check(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= C,
+           "conv_rotate_store: the projection must be float32 [T, >= C]")
+    _check(taps.dim() == 2 and taps.shape[0] == C and 1 <= K <= CONV_MAX_TAPS, f"conv_rotate_store: taps must be [{C}, up to {CONV_MAX_TAPS}]")
+    _f32(taps, "conv_rotate_store taps")
+    _check(state.dtype == torch.float32 and offset + (K - 1) * C <= state.shape[1], "conv_rotate_store: the kept inputs do not fit the state")
+    rot = 0
+    if freq is not None:
+        _f32(freq, "conv_rotate_store freq")
+        rot = 2 * freq.numel()
+        _check(rot <= dim, f"conv_rotate_store: rotary width {rot} exceeds the head size {dim}")
+    page = 0
+    if k_heads:
+        _check(v_heads > 0 and k_cache is not None and v_cache is not None and slots is not None, "conv_rotate_store: keys and values need their caches")
+        _check_caches(k_cache, v_cache, out_dtype, k_heads, head_size, "conv_rotate_store")
+        _check(v_heads * v_repeat == k_heads, "conv_rotate_store: the value cache has one head per key head")
+        _i32(slots, "slots", T)
+        page = k_cache.shape[1]
+    else:
+        _check(v_heads == 0, "conv_rotate_store: values come with keys")
+    _i32(ctx.pos, "pos", T)
+    q = (torch.empty if head_size == dim else torch.zeros)(T, heads * head_size, dtype=out_dtype, device=proj.device)
+    kept, stride = _state_ptr(state, offset)
+    one_launch = ctx.facts.decode_only and T == ctx.num_seqs and (rot == 0 or dim % 2 == 0)
+    _call("tl_conv_rotate_store", _ptr(proj), proj.stride(0) if T > 1 else max(C, proj.stride(0)), _ptr(taps), kept,
+          ctypes.c_longlong(stride), _ptr(ctx.state_slots), _ptr(ctx.seq_of_token), _ptr(ctx.q_start), _ptr(ctx.pos), _ptr(freq),
+          ctypes.c_float(mag), rot, _ptr(slots) if k_heads else _ptr(None), _ptr(q), _ptr(k_cache) if k_heads else _ptr(None),
+          _ptr(v_cache) if k_heads else _ptr(None), _code(q, "conv_rotate_store"), T, ctx.num_seqs, heads, k_heads, dim, v_heads,
+          vdim, head_size, max(v_repeat, 1), page, K, 2 if one_launch else 1, _stream())
+    return q
+
+
+def diff_combine(a: torch.Tensor, heads: int, kv_heads: int, vdim: int, head_size: int, lam: float, eps: float,
+                 post: float) -> torch.Tensor:
+    """The two maps of differential attention put together: ``a`` [T, 2 * heads * head_size] is what attention leaves
+    for the maps as query heads ordered (key/value head g, map m, place r in the group): head ``(2 g + m) R + r``, R =
+    heads / kv_heads, is map m of head ``g R + r``; its first ``vdim`` columns count.  Returns [T, heads * vdim]:
+    ``(a1 - lam * a2) / sqrt(mean((a1 - lam * a2)^2) + eps) * post`` per head, float32 arithmetic."""
+    _on_gpu(a)
+    T = a.shape[0]
+    _check(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == 2 * heads * head_size and heads % kv_heads == 0 and vdim <= head_size,
+           "diff_combine: bad shapes")
+    out = torch.empty(T, heads * vdim, dtype=a.dtype, device=a.device)
+    _call("tl_diff_combine", _ptr(a), a.stride(0) if T > 1 else a.shape[1], _ptr(out), _code(a, "diff_combine"), T, heads, kv_heads,
+          vdim, head_size, ctypes.c_float(lam), ctypes.c_float(eps), ctypes.c_float(post), _stream())
+    return out

@@ -141,3 +141,63 @@ class PreNormTokenInputBlock:
         if self.token_input is not None:
             y = self.token_input.forward(x, y, ctx)
         return y
+
+
+@register_block("sandwich")
+class SandwichBlock:
+    """Every branch is normed on both sides: its input by a pre-norm, its output by a second norm before it
+    joins the stream with a factor ``m`` (``LayerSpec.branch_scale``):
+
+        x <- x + m * post1(mixer(norm1(x)));  [x <- x + m * post2(ffn(norm2(x)))]
+
+    The feed-forward with its two norms may be absent.  A branch's normed output is not added at once: it is
+    handed on as :class:`tensorline_amd.ops.kernels.NormedBranch`, and the norm that reads the stream next (this
+    block's second pre-norm, the next block's first, the final norm) norms it, adds it and norms the sum in one
+    pass.  Where whoever runs next does not take that form (``after.normed_branch``), the block adds it itself
+    and leaves nothing."""
+
+    def __init__(self, spec: LayerSpec, hidden_size: int, dtype, device):
+        common = dict(hidden_size=hidden_size, dtype=dtype, device=device)
+        self.spec = spec
+        self.scale = float(spec.branch_scale)
+        if spec.mixer_post_norm is None or (spec.feed_forward is not None and spec.feed_forward_post_norm is None):
+            raise ValueError(f"{spec.prefix}: a sandwich block needs a norm behind every branch")
+        self.mixer_norm = build_part("norm", spec.mixer_norm, layer_prefix=spec.prefix, **common)
+        self.mixer = build_part("mixer", spec.mixer, layer_prefix=spec.prefix, **common)
+        self.mixer_post = build_part("norm", spec.mixer_post_norm, layer_prefix=spec.prefix, **common)
+        self.feed_forward_norm = self.feed_forward = self.feed_forward_post = None
+        if spec.feed_forward is not None:
+            self.feed_forward_norm = build_part("norm", spec.feed_forward_norm, layer_prefix=spec.prefix, **common)
+            self.feed_forward = build_part("feed_forward", spec.feed_forward, layer_prefix=spec.prefix, **common)
+            self.feed_forward_post = build_part("norm", spec.feed_forward_post_norm, layer_prefix=spec.prefix, **common)
+        for norm in (self.mixer_post, self.feed_forward_post):
+            if norm is not None and not hasattr(norm, "as_branch"):
+                raise ValueError(f"{spec.prefix}: the norm behind a branch must offer as_branch (an RMS norm does)")
+        if self.feed_forward_norm is not None and not getattr(self.feed_forward_norm, "adds_normed_branch", False):
+            raise ValueError(f"{spec.prefix}: the feed-forward's pre-norm must take a normed branch as its residual")
+
+    def parts(self) -> list[Part]:
+        return [p for p in (self.mixer_norm, self.mixer, self.mixer_post, self.feed_forward_norm, self.feed_forward,
+                            self.feed_forward_post) if p is not None]
+
+    def cache_need(self):
+        fn = getattr(self.mixer, "cache_need", None)
+        return fn() if fn is not None else None
+
+    def state_need(self):
+        fn = getattr(self.mixer, "state_need", None)
+        return fn() if fn is not None else None
+
+    def intake(self) -> Intake:
+        return Intake(None, False, bool(getattr(self.mixer_norm, "adds_normed_branch", False)))
+
+    def forward(self, x: torch.Tensor, carry, ctx, cache, after: Intake | None = None):
+        y = self.mixer.forward(self.mixer_norm.forward(x, carry), ctx, cache)
+        branch = self.mixer_post.as_branch(y, self.scale)
+        if self.feed_forward is not None:
+            y = self.feed_forward.forward(self.feed_forward_norm.forward(x, branch), ctx)
+            branch = self.feed_forward_post.as_branch(y, self.scale)
+        if after is not None and after.normed_branch:
+            return branch
+        kernels.add_normed_branch(x, branch)
+        return None

@@ -2,7 +2,9 @@
 the head that turns normed rows into logits.
 
 * **Embedding** (``@register_embedding``): ``forward(ids int32 [T]) -> float32 [T, H]``.  One that a
-  head may be tied to exposes ``name`` (its tensor's checkpoint name) and ``table`` ([V, H]).
+  head may be tied to exposes ``name`` (its tensor's checkpoint name) and ``table`` ([V, H]).  One that
+  looks at more than the ids has ``forward_step(ctx)`` instead, and ``state_need()`` if it keeps something
+  per request (found in ``ctx.input_state``, indexed by ``ctx.state_slots``).
 * **Head** (``@register_head``): ``load(get, embedding)``, ``optional_tensors(embedding)`` (names a
   checkpoint may hold besides the declared ones, each with the declared tensor it must equal),
   ``forward(h) -> float32 logits [R, V]`` for the wanted rows only, and ``takes_normed_rows()``:
@@ -20,7 +22,7 @@ import torch
 from tensorline_amd.ops import kernels
 from tensorline_amd.parts.base import Linear, Part, TensorGetter
 from tensorline_amd.parts.registry import register_embedding, register_head
-from tensorline_amd.parts.spec import TensorDecl
+from tensorline_amd.parts.spec import StateNeed, TensorDecl
 
 
 @register_embedding("token_embedding")
@@ -47,6 +49,47 @@ class TokenEmbedding(Part):
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
         return kernels.embed(ids, self.table, scale=self.scale)
+
+
+@register_embedding("bigram_embedding")
+class BigramEmbedding(TokenEmbedding):
+    """The token's row plus a row of a second table picked by a hash of (token before, token):
+    ``(prev * mul_prev + token * mul_cur) mod buckets``; a sequence's first token reads the table's last row,
+    number ``buckets``.  The token before the step's first is per-request state: an int32 in the request's
+    slot, kept by the cache manager like a mixer's state (zeroed with the slot; position 0 never reads it).
+    Tensors: ``name`` [vocab, hidden], ``bigram_name`` [buckets + 1, hidden].  The sum is float32."""
+
+    def __init__(self, hidden_size, prefix, dtype, device, vocab_size: int, name: str, bigram_name: str, buckets: int,
+                 mul_prev: int, mul_cur: int, std: float = 0.02):
+        super().__init__(hidden_size, prefix, dtype, device, vocab_size, name, std)
+        self.bigram_name = prefix + bigram_name
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        if self.buckets <= 0:
+            raise ValueError(f"{self.bigram_name}: the number of buckets must be positive")
+        self.bigram: torch.Tensor | None = None
+
+    def tensors(self):
+        return {**super().tensors(),
+                self.bigram_name: TensorDecl((self.buckets + 1, self.hidden_size), "normal", self.std, "compute")}
+
+    def load(self, get: TensorGetter) -> None:
+        super().load(get)
+        self.bigram = get(self.bigram_name)
+
+    def weight_tensors(self):
+        return [self.table, self.bigram]
+
+    def state_need(self) -> StateNeed:
+        return StateNeed((1,), "int32")
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        raise TypeError("the bigram embedding needs the step's context: forward_step(ctx)")
+
+    def forward_step(self, ctx) -> torch.Tensor:
+        if ctx.input_state is None:
+            raise ValueError("the bigram embedding keeps the token before per request: the cache manager must be "
+                             "built with the model's input_state_need()")
+        return kernels.embed_bigram(ctx.ids, ctx, self.table, self.bigram, ctx.input_state, self.mul_prev, self.mul_cur)
 
 
 @register_head("lm_head")

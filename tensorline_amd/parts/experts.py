@@ -5,8 +5,10 @@
     expert(h) = W_down (g * sigmoid(alpha g) * (u + 1)),  g = min(W_gate h, limit),  u = clamp(W_up h, +-limit)
 
 Other designs change the weights (``weighting`` "sigmoid": each chosen expert by its own score,
-``router_scale * sigmoid(z_e)``, not renormalised), leave the router without bias, or use the plain
-gated activation ``silu(g) * u`` (``activation`` "swiglu": no limit, alpha 1, nothing added to u).
+``router_scale * sigmoid(z_e)``, not renormalised; "softmax_all": the chosen experts' shares of the
+softmax over all experts, not renormalised), leave the router without bias, use the plain gated
+activation ``silu(g) * u`` (``activation`` "swiglu": no limit, alpha 1, nothing added to u), or have
+experts without gate, ``W_down relu(W_up h)^2`` (``activation`` "relu2": tensors e<i>.up / .down only).
 
 The experts' matrices are stacked ([experts, 2 ff, width] gate over up, [experts, width, ff]); a
 step's (token, choice) pairs are ordered by expert on the device and both products run as one
@@ -27,17 +29,18 @@ from tensorline_amd.parts.spec import TensorDecl
 @register_feed_forward("routed_experts")
 class RoutedExperts(Part):
     """Parameters: ``experts``, ``top``, ``ff`` and ``limit`` of an expert, ``shared`` = {ff, limit} or
-    None, ``alpha`` of the gate's sigmoid; ``weighting`` ("softmax_top" or "sigmoid"), ``router_scale``,
-    ``router_bias``, ``activation`` ("clamped_glu" or "swiglu").  Tensors under the prefix: router,
+    None, ``alpha`` of the gate's sigmoid; ``weighting`` ("softmax_top", "sigmoid" or "softmax_all"),
+    ``router_scale``, ``router_bias``, ``activation`` ("clamped_glu", "swiglu" or "relu2").  Tensors under the prefix: router,
     router.b, e<i>.gate / .up / .down, shared.gate / .up / .down."""
 
     def __init__(self, hidden_size, prefix, dtype, device, experts: int, top: int, ff: int, limit: float | None = None,
                  shared: dict | None = None, alpha: float = 1.702, weighting: str = "softmax_top", router_scale: float = 1.0,
                  router_bias: bool = True, activation: str = "clamped_glu"):
         super().__init__(hidden_size, prefix, dtype, device)
-        if activation not in ("clamped_glu", "swiglu") or weighting not in ("softmax_top", "sigmoid"):
+        if activation not in ("clamped_glu", "swiglu", "relu2") or weighting not in kernels.ROUTER_WEIGHTINGS:
             raise ValueError(f"{prefix}: unknown activation {activation!r} or weighting {weighting!r}")
-        if activation == "swiglu":
+        self.gated = activation != "relu2"
+        if activation in ("swiglu", "relu2"):
             limit, alpha, self.shift = float("inf"), 1.0, 0.0
         else:
             if limit is None:
@@ -65,7 +68,8 @@ class RoutedExperts(Part):
         out = dict(self.router.tensors())
         for e in range(self.experts):
             p = f"{self.prefix}e{e}."
-            out[p + "gate"] = TensorDecl((self.ff, self.hidden_size), "normal", 0.05, "compute")
+            if self.gated:
+                out[p + "gate"] = TensorDecl((self.ff, self.hidden_size), "normal", 0.05, "compute")
             out[p + "up"] = TensorDecl((self.ff, self.hidden_size), "normal", 0.05, "compute")
             out[p + "down"] = TensorDecl((self.hidden_size, self.ff), "normal", 0.05, "compute")
         if self.shared_down is not None:
@@ -77,7 +81,10 @@ class RoutedExperts(Part):
         self.router.load(get)
         self.router.prepare()
         name = lambda e, s: f"{self.prefix}e{e}.{s}"
-        self.gate_up = torch.stack([torch.cat([get(name(e, "gate")), get(name(e, "up"))]) for e in range(self.experts)]).contiguous()
+        if self.gated:
+            self.gate_up = torch.stack([torch.cat([get(name(e, "gate")), get(name(e, "up"))]) for e in range(self.experts)]).contiguous()
+        else:
+            self.gate_up = torch.stack([get(name(e, "up")) for e in range(self.experts)]).contiguous()
         self.down = torch.stack([get(name(e, "down")) for e in range(self.experts)]).contiguous()
         if self.shared_down is not None:
             self._sg.load(get)
@@ -104,4 +111,5 @@ class RoutedExperts(Part):
         if self.shared_down is not None:
             act = kernels.clamp_glu(self.shared_gate_up(h, out_dtype=torch.float32), self.shared_limit, self.alpha, self.dtype)
             shared = self.shared_down(act, out_dtype=torch.float32)
-        return kernels.moe_experts(h, self.gate_up, self.down, ids, weights, self.limit, self.alpha, shared, self.shift)
+        return kernels.moe_experts(h, self.gate_up, self.down, ids, weights, self.limit, self.alpha, shared, self.shift,
+                                   gated=self.gated)

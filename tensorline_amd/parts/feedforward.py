@@ -16,13 +16,16 @@ from tensorline_amd.parts.registry import register_feed_forward
 
 @register_feed_forward("swiglu")
 class SwiGLU(Part):
-    def __init__(self, hidden_size, prefix, dtype, device, intermediate_size: int):
+    def __init__(self, hidden_size, prefix, dtype, device, intermediate_size: int, names: tuple | None = None):
+        """``names``: the checkpoint names of the gate, up and down matrices below the prefix where they are
+        not ``gate_proj.weight``, ``up_proj.weight`` and ``down_proj.weight``."""
         super().__init__(hidden_size, prefix, dtype, device)
         self.intermediate_size = int(intermediate_size)
-        self._gate = Linear(prefix + "gate_proj", hidden_size, self.intermediate_size, False)
-        self._up = Linear(prefix + "up_proj", hidden_size, self.intermediate_size, False)
+        g, u, d = (prefix + n for n in names) if names else (None, None, None)
+        self._gate = Linear(prefix + "gate_proj", hidden_size, self.intermediate_size, False, weight_name=g)
+        self._up = Linear(prefix + "up_proj", hidden_size, self.intermediate_size, False, weight_name=u)
         self.gate_up: Linear | None = None
-        self.down = Linear(prefix + "down_proj", self.intermediate_size, hidden_size, False)
+        self.down = Linear(prefix + "down_proj", self.intermediate_size, hidden_size, False, weight_name=d)
 
     def tensors(self):
         return {**self._gate.tensors(), **self._up.tensors(), **self.down.tensors()}

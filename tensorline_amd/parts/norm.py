@@ -32,6 +32,11 @@ class RMSNorm(Part):
         return [self.weight]
 
     adds_share_sums = True
+    adds_normed_branch = True      # ``forward`` takes a kernels.NormedBranch as the residual
+
+    def as_branch(self, y: torch.Tensor, mult: float) -> "kernels.NormedBranch":
+        """``mult * norm(y)``, left for the norm that reads the stream next to add in its own pass."""
+        return kernels.NormedBranch(y, self.weight, self.eps, float(mult))
 
     def deferrable(self) -> tuple[torch.Tensor, float]:
         """(weight, eps): all a product needs to carry this norm (see ``Part.defers_norm``)."""

@@ -50,6 +50,10 @@ class LayerSpec:
     feed_forward_norm: PartSpec | None
     block: str = "prenorm"            # the arrangement of the parts
     token_input: PartSpec | None = None   # a per-layer input from the token ids, for blocks that take one
+    # for blocks that norm a branch's output before it joins the stream: those norms, and the factor on the normed output
+    mixer_post_norm: PartSpec | None = None
+    feed_forward_post_norm: PartSpec | None = None
+    branch_scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -65,9 +69,12 @@ class Intake:
     told the intake of its successor and may answer with the cheaper form.
     ``normed_rows_for``: (weight, eps) of the norm the successor applies first, if it takes that
     norm's input as ``tensorline_amd.ops.kernels.NormedRows``.  ``share_sums``: its first norm adds a
-    product left in its shares of K (``tensorline_amd.ops.kernels.ShareSum``)."""
+    product left in its shares of K (``tensorline_amd.ops.kernels.ShareSum``).  ``normed_branch``: its
+    first norm adds a branch output that is still to be normed and scaled
+    (``tensorline_amd.ops.kernels.NormedBranch``)."""
     normed_rows_for: tuple | None = None
     share_sums: bool = False
+    normed_branch: bool = False
 
 
 @dataclass(frozen=True)
