@@ -483,6 +483,47 @@ def make_tumitar_twin(size: str):
         rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768))
 
 
+# ---- the Zeganex design beside the dense decoder at equal size ----------------------------------------
+# Layer sizes that resemble real models of its kinds: rotary layers with heads of 128 in groups of four, half of a
+# head rotated, an output gate; two-map layers with half as many heads, maps of 64 and values of 128; convolutions of
+# four taps; windows of 4,096 tokens (beyond the contexts measured, so that attention does the dense model's work);
+# a SwiGLU of three widths, experts without gate of which 6 are used.  Four layers (rotary + dense, two maps +
+# experts, rotary + experts, two maps reading the second layer's cache + experts).  ``dense`` has the same width,
+# layers, vocabulary and attention heads, and a SwiGLU with the mean of the feed-forward weights a token reads.
+ZEGANEX_SIZES = {
+    "w1024": dict(width=1024, heads=8, experts=32, top=6, ff=512),
+    "w2048": dict(width=2048, heads=16, experts=64, top=6, ff=1408),
+    "w4096": dict(width=4096, heads=32, experts=64, top=6, ff=2048),
+}
+
+
+def make_zeganex_config(size: str):
+    from tensorline_amd.config import ZeganexConfig
+    z = ZEGANEX_SIZES[size]
+    W, H = z["width"], z["heads"]
+    rotary = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4, "mask": {"size": 4096},
+              "rot": {"dims": 64, "base": 10000.0, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    maps = {"heads": H // 2, "kv_heads": max(1, H // 8), "dim": 64, "vdim": 128, "scale": 64 ** -0.5, "conv": 4, "diff": 0.5,
+            "mask": {"size": 4096}}
+    moe = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"]}, "expert": {"ff": z["ff"]}}
+    dense = {"kind": "dense", "ff": 3 * W}
+    layers = [{"type": "attention_2", "mixer": rotary, "mlp": dense}, {"type": "attention", "mixer": maps, "mlp": moe},
+              {"type": "attention_2", "mixer": rotary, "mlp": moe}, {"type": "attention", "mixer": {**maps, "kv_from": 1}, "mlp": moe}]
+    return ZeganexConfig.from_dict({"architecture": "Zeganex", "vocab": HYBRID_VOCAB, "width": W, "norm": {"eps": 1e-6},
+                                    "residual_mult": 0.5, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 8191, "mul_cur": 31}},
+                                    "layers": layers})
+
+
+def make_zeganex_twin(size: str):
+    from tensorline_amd.config import Qwen2Config
+    z = ZEGANEX_SIZES[size]
+    inter = (3 * 3 * z["width"] + 3 * 2 * z["top"] * z["ff"]) // (4 * 3) // 128 * 128
+    return Qwen2Config.from_dict(dict(
+        architectures=["Qwen2ForCausalLM"], vocab_size=HYBRID_VOCAB, hidden_size=z["width"], intermediate_size=inter,
+        num_hidden_layers=4, num_attention_heads=z["heads"], num_key_value_heads=max(1, z["heads"] // 4), head_dim=128,
+        rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768))
+
+
 def profile_step(llm, entries_of, seed: int) -> dict:
     """Event time of every kernel of one eager step, summed per entry point (milliseconds), after a
     warm-up step of the same shape."""
@@ -513,7 +554,7 @@ def profile_step(llm, entries_of, seed: int) -> dict:
 
 def bench_hybrid(args, design: str = "samovik") -> int:
     """Prefill and decode throughput of a design at real layer sizes (``samovik``: HYBRID_SIZES, ``tumitar``:
-    TUMITAR_SIZES) beside the dense decoder at equal size, and each step's time by kernel.  One JSON line;
+    TUMITAR_SIZES, ``zeganex``: ZEGANEX_SIZES) beside the dense decoder at equal size, and each step's time by kernel.  One JSON line;
     the default benchmark is not run."""
     import torch
     table, make, make_twin, model_text = {
@@ -522,7 +563,10 @@ def bench_hybrid(args, design: str = "samovik") -> int:
                     "Qwen2 layers of equal width (4 layers)"),
         "tumitar": (TUMITAR_SIZES, make_tumitar_config, make_tumitar_twin,
                     "Tumitar layer sizes (4 layers: parallel + dense, parallel + experts, rglru + dense, parallel + experts) "
-                    "beside Qwen2 layers of equal width (4 layers)")}[design]
+                    "beside Qwen2 layers of equal width (4 layers)"),
+        "zeganex": (ZEGANEX_SIZES, make_zeganex_config, make_zeganex_twin,
+                    "Zeganex layer sizes (4 layers: rotary attention + dense, two-map attention + experts, rotary attention + "
+                    "experts, two-map attention on the second layer's cache + experts) beside Qwen2 layers of equal width (4 layers)")}[design]
 
     from tensorline_amd import LLM
     from tensorline_amd.engine.batch import StepEntry
@@ -611,6 +655,9 @@ def main() -> int:
     ap.add_argument("--tumitar", action="store_true",
                     help="the same for the Tumitar design (attention beside a state-space mixer, gated recurrent layers, dense "
                          "and routed feed-forwards)")
+    ap.add_argument("--zeganex", action="store_true",
+                    help="the same for the Zeganex design (attention with short convolutions in two kinds, norms on both sides "
+                         "of every branch, experts without gate)")
     ap.add_argument("--hybrid-sizes", default="", help="which of w1024,w2048,w4096 (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -622,6 +669,8 @@ def main() -> int:
         return bench_hybrid(args)
     if args.tumitar:
         return bench_hybrid(args, "tumitar")
+    if args.zeganex:
+        return bench_hybrid(args, "zeganex")
 
     import torch
 

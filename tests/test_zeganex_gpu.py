@@ -11,7 +11,7 @@ import torch
 
 from tests import plain_zeganex as P
 from tests.helpers import steps_portions, steps_prefill_then_decode, steps_whole
-from tests.samovik_helpers import LIMIT, rel_error, run_steps
+from tests.samovik_helpers import rel_error, run_steps
 from tests.test_samovik_gpu import mixed_steps
 from tests.tumitar_helpers import run_steps_with_routes
 from tests.zeganex_helpers import (CFG_A, CFG_B, CFG_C, CONFIGS, YARN, _dense, _moe, _rotary, _two_maps, build, one_layer,
@@ -20,6 +20,10 @@ from tests.zeganex_helpers import (CFG_A, CFG_B, CFG_C, CONFIGS, YARN, _dense, _
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 DTYPES = ["float32", "bfloat16"]
+# Of the logits' own root mean square.  Every branch output is normed to unit size before it joins the stream, so the
+# rounding of a narrow random model is not damped on its way through the layers (a subtraction of two rounded maps,
+# normed again, among it); every case that bfloat16 runs, float32 runs too, at a thousandth of the limit.
+LIMIT = {"float32": 2e-5, "bfloat16": 6e-2}
 
 
 def tokens_for(cfg, n, seed):
@@ -446,15 +450,12 @@ def test_tokens_far_back_reach_the_end_through_the_layers(dtype):
     cfg = CFG_C
     model, w = build(cfg, dtype, seed=8)
     toks = tokens_for(cfg, 400, 7)
-    want = P.forward(w, cfg, toks).numpy()
     steps, at = [], 0
     for n in [150, 130, 2, 60, 26] + [1] * 32:
-        steps.append({"entries": [{"id": "a", "tokens": toks[at:at + n], "want": [n - 1]}], "end": ["a"] if at + n == len(toks) else []})
+        steps.append({"entries": [{"id": "a", "tokens": toks[at:at + n], "want": list(range(n))}], "end": ["a"] if at + n == len(toks) else []})
         at += n
     assert at == len(toks)
-    got = run_steps(model, steps, max_tokens=448)["a"]
-    for p, row in got.items():
-        assert rel_error(row, want[p]) < LIMIT[dtype], f"position {p}: {rel_error(row, want[p]):.3e}"
+    run_and_check(model, steps, cfg, w, {"a": toks}, dtype, "400 tokens", max_tokens=448)
 
 
 # ---- long decoding, graphs, the entry point ------------------------------------------------------------------
@@ -468,8 +469,13 @@ def test_long_decoding_eager_and_from_graphs(dtype):
         entries = [{"id": r, "tokens": [t[i]], "want": [0]} for r, t in reqs.items() if i < len(t)]
         steps.append({"entries": entries, "end": [r for r, t in reqs.items() if i == len(t) - 1]})
     run_and_check(model, copy.deepcopy(steps), cfg, w, reqs, dtype, "long decoding", max_tokens=512)
-    eager = run_steps(model, copy.deepcopy(steps), max_tokens=512)
-    replayed = run_steps(model, copy.deepcopy(steps), max_tokens=512, graphs=True)
+    # a replayed step computes what its eager twin computes, when both split a context's keys for the same longest context
+    from tensorline_amd.engine.replay import TraceSession
+    plain_session, graph_session = TraceSession(model, 512), TraceSession(model, 512, graphs=True)
+    plain_session.runner.fit_context = graph_session.runner.fit_context
+    eager = run_steps(model, copy.deepcopy(steps), session=plain_session)
+    replayed = run_steps(model, copy.deepcopy(steps), session=graph_session)
+    assert graph_session.runner.graph_replays > 100
     for rid, toks in reqs.items():
         for p in range(len(toks)):
             assert rel_error(replayed[rid][p], eager[rid][p]) < 1e-6, f"{rid} at {p}: a graph's step differs from the eager one"
