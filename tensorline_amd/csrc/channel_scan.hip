@@ -301,6 +301,90 @@ __global__ __launch_bounds__(256) void conv_rotate_store_kernel(
         v_cache[((pg * Gv * v_rep + (size_t)head * v_rep + r) * D + i) * page + within] = tl_from_float<O>(y);
 }
 
+// The same with four neighbouring channels per thread, for head sizes that are multiples of four and rows that start
+// at 16-byte borders: 16-byte loads of the projection and the kept inputs; a work-group computes the token's cosines
+// and sines once (rot / 2 of them, in LDS) for all its heads; a rotated pair lies within its thread, so nothing is
+// computed twice and the one-launch form needs no barrier.
+template <typename O>
+__device__ __forceinline__ void crs_store4(O* p, float4 v);
+template <>
+__device__ __forceinline__ void crs_store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <>
+__device__ __forceinline__ void crs_store4<bf16_t>(bf16_t* p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)tl_f2bf_bits(v.x) | ((uint32_t)tl_f2bf_bits(v.y) << 16);
+    u.y = (uint32_t)tl_f2bf_bits(v.z) | ((uint32_t)tl_f2bf_bits(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+
+template <typename O>
+__global__ __launch_bounds__(256) void conv_rotate_store_vec_kernel(
+    const float* __restrict__ proj, int ldp, const float* __restrict__ taps, float* __restrict__ kept, long long state_stride,
+    const int32_t* __restrict__ state_slots, const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ pos, const float* __restrict__ freq, float mag, int rot, const int32_t* __restrict__ slots,
+    O* __restrict__ q_out, O* __restrict__ k_cache, O* __restrict__ v_cache, int Hq, int Gk, int d, int Gv, int dv, int D,
+    int v_rep, int page, int C, int K, int shift) {
+    __shared__ float cs_s[128], sn_s[128];          // one cosine and sine per rotated pair of the token, times mag
+    const int t = blockIdx.x;
+    if (freq != nullptr) {
+        const float p = (float)pos[t];
+        for (int i = threadIdx.x; i < (rot >> 1); i += blockDim.x) {
+            float sn, cs;
+            sincosf(p * freq[i], &sn, &cs);
+            sn_s[i] = sn * mag;
+            cs_s[i] = cs * mag;
+        }
+        __syncthreads();
+    }
+    const int s = seq_of_token[t];
+    const int r0 = q_start[s];
+    float* old = kept + (size_t)state_slots[s] * state_stride;
+    const int slot = slots ? slots[t] : -1;
+    const int qk = (Hq + Gk) * d;
+  for (int c = 4 * (blockIdx.y * blockDim.x + threadIdx.x); c < C; c += 4 * blockDim.x * gridDim.y) {
+    const float* tp = taps + (size_t)c * K;             // the four channels' taps, 4 K floats in a row
+    float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j = 0; j < K; ++j) {
+        const int r = t - (K - 1) + j;
+        const float4 v = r >= r0 ? *reinterpret_cast<const float4*>(proj + (size_t)r * ldp + c)
+                                 : *reinterpret_cast<const float4*>(old + (size_t)(r - r0 + K - 1) * C + c);
+        y.x += tp[j] * v.x;
+        y.y += tp[K + j] * v.y;
+        y.z += tp[2 * K + j] * v.z;
+        y.w += tp[3 * K + j] * v.w;
+        if (shift && j > 0) *reinterpret_cast<float4*>(old + (size_t)(j - 1) * C + c) = v;
+    }
+    if (c < qk) {
+        const int head = c / d, i = c - head * d;
+        if (freq != nullptr && i < rot) {
+            float sn = sn_s[i >> 1], cs = cs_s[i >> 1];
+            const float a = y.x, b = y.y;
+            y.x = a * cs - b * sn;
+            y.y = b * cs + a * sn;
+            if (i + 2 < rot) {
+                sn = sn_s[(i >> 1) + 1];
+                cs = cs_s[(i >> 1) + 1];
+                const float a2 = y.z, b2 = y.w;
+                y.z = a2 * cs - b2 * sn;
+                y.w = b2 * cs + a2 * sn;
+            }
+        }
+        if (head < Hq) crs_store4<O>(q_out + ((size_t)t * Hq + head) * D + i, y);
+        else if (slot >= 0) crs_store4<O>(k_cache + ((size_t)slot * Gk + (head - Hq)) * D + i, y);
+        continue;
+    }
+    if (slot < 0) continue;
+    const int head = (c - qk) / dv, i = (c - qk) - head * dv;
+    const size_t pg = (size_t)slot / page, within = (size_t)slot % page;
+    const float vals[4] = {y.x, y.y, y.z, y.w};
+    for (int r = 0; r < v_rep; ++r) {
+        O* base = v_cache + ((pg * Gv * v_rep + (size_t)head * v_rep + r) * D + i) * page + within;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) base[(size_t)e * page] = tl_from_float<O>(vals[e]);
+    }
+  }
+}
+
 // update: 1 renews the kept inputs by a second launch, 2 in the same launch (steps of one token per
 // sequence, T == S; needs rot == 0 or an even d, so that a pair's channels lie in one work-group).
 extern "C" int tl_conv_rotate_store(const float* proj, int ldp, const float* taps, float* kept, long long state_stride,
@@ -324,6 +408,26 @@ extern "C" int tl_conv_rotate_store(const float* proj, int ldp, const float* tap
     if (T == 0 || S == 0) return 0;
     if (rot == 0) freq = nullptr;
     const int shift = update == 2 ? 1 : 0;
+    const bool vec = rot <= 256 && d % 4 == 0 && dv % 4 == 0 && D % 4 == 0 && ldp % 4 == 0 && (uintptr_t)proj % 16 == 0 && (uintptr_t)kept % 16 == 0 &&
+                     state_stride % 4 == 0 && (uintptr_t)q_out % 16 == 0 && (uintptr_t)k_cache % 16 == 0;
+    if (vec && (dtype == TL_F32 || dtype == TL_BF16)) {
+        dim3 vblock(256), vgrid(T, tl_ceil_div(C, 1024));
+        if (dtype == TL_F32)
+            hipLaunchKernelGGL(conv_rotate_store_vec_kernel<float>, vgrid, vblock, 0, stream, proj, ldp, taps, kept, state_stride,
+                               state_slots, seq_of_token, q_start, pos, freq, mag, rot, slots, (float*)q_out, (float*)k_cache,
+                               (float*)v_cache, Hq, Gk, d, Gv, dv, D, v_rep, page, C, K, shift);
+        else
+            hipLaunchKernelGGL(conv_rotate_store_vec_kernel<bf16_t>, vgrid, vblock, 0, stream, proj, ldp, taps, kept, state_stride,
+                               state_slots, seq_of_token, q_start, pos, freq, mag, rot, slots, (bf16_t*)q_out, (bf16_t*)k_cache,
+                               (bf16_t*)v_cache, Hq, Gk, d, Gv, dv, D, v_rep, page, C, K, shift);
+        TL_CHECK_LAUNCH("tl_conv_rotate_store");
+        if (update == 1 && K > 1) {
+            hipLaunchKernelGGL(causal_conv_keep_kernel, dim3(tl_ceil_div(C, 256), S), dim3(256), 0, stream, proj, ldp, kept,
+                               state_stride, state_slots, q_start, C, K);
+            TL_CHECK_LAUNCH("tl_conv_rotate_store keep");
+        }
+        return 0;
+    }
     dim3 block(256), grid(T, tl_ceil_div(C, 256));
     if (dtype == TL_F32)
         hipLaunchKernelGGL(conv_rotate_store_kernel<float>, grid, block, 0, stream, proj, ldp, taps, kept, state_stride, state_slots,

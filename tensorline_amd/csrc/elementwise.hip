@@ -119,66 +119,6 @@ extern "C" int tl_embed_bigram(const int32_t* ids, const int32_t* pos, const int
     return 0;
 }
 
-// ---- a normed branch added to the stream, and the next norm -------------------------------------
-// A residual branch whose output y is RMS-normed before it joins the stream:
-//   x[r] += mult * y[r] / sqrt(mean(y[r]^2) + eps_b) * wb
-// and, with w, the norm that reads the stream next, out[r] = x[r] / sqrt(mean(x[r]^2) + eps) * w, in the
-// same pass.  With `rows`: out only, for x[rows[r]] and y[rows[r]]; x is left as it is.  Float sums.
-template <typename O, bool HAS_ROWS>
-__global__ __launch_bounds__(1024) void branch_norm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
-                                                               const float* __restrict__ wb, float mult, float eps_b,
-                                                               const float* __restrict__ w, float eps, O* __restrict__ out,
-                                                               const int32_t* __restrict__ rows, int H) {
-    __shared__ float red[16];
-    const int r = blockIdx.x;
-    const size_t src = HAS_ROWS ? (size_t)rows[r] : (size_t)r;
-    float* xr = x + src * H;
-    const float* yr = y + src * H;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) ss += yr[c] * yr[c];
-    ss = tl_block_sum(ss, red);
-    const float f = mult / sqrtf(ss / (float)H + eps_b);
-    float sx = 0.f;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) {
-        const float v = xr[c] + yr[c] * f * wb[c];
-        if (!HAS_ROWS) xr[c] = v;
-        sx += v * v;
-    }
-    if (!w) return;
-    sx = tl_block_sum(sx, red);
-    const float rstd = 1.0f / sqrtf(sx / (float)H + eps);
-    O* orow = out + (size_t)r * H;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) {
-        const float v = HAS_ROWS ? xr[c] + yr[c] * f * wb[c] : xr[c];
-        orow[c] = tl_from_float<O>(v * rstd * w[c]);
-    }
-}
-
-extern "C" int tl_branch_norm_add(float* x, const float* y, const float* wb, float mult, float eps_b, const float* w, float eps,
-                                  void* out, int out_dtype, const int32_t* rows, int n_rows, int H, hipStream_t stream) {
-    TL_CHECK_ARG(n_rows >= 0 && H > 0 && eps >= 0.f && eps_b >= 0.f, "tl_branch_norm_add: bad sizes rows=%d H=%d", n_rows, H);
-    TL_CHECK_ARG((w == nullptr) == (out == nullptr) && (rows == nullptr || w != nullptr), "tl_branch_norm_add: a norm needs its output, and rows a norm");
-    if (n_rows == 0) return 0;
-    int threads = ((H + 63) / 64) * 64;
-    if (threads > 1024) threads = 1024;
-    dim3 grid(n_rows), block(threads);
-#define TL_BRANCH_CASE(OT)                                                                                                       \
-    do {                                                                                                                         \
-        if (rows)                                                                                                                \
-            hipLaunchKernelGGL((branch_norm_add_kernel<OT, true>), grid, block, 0, stream, x, y, wb, mult, eps_b, w, eps, (OT*)out, \
-                               rows, H);                                                                                         \
-        else                                                                                                                     \
-            hipLaunchKernelGGL((branch_norm_add_kernel<OT, false>), grid, block, 0, stream, x, y, wb, mult, eps_b, w, eps,          \
-                               (OT*)out, rows, H);                                                                               \
-    } while (0)
-    if (out_dtype == TL_BF16) TL_BRANCH_CASE(bf16_t);
-    else if (out_dtype == TL_F32) TL_BRANCH_CASE(float);
-    else return tl_fail("tl_branch_norm_add: unknown dtype %d", out_dtype);
-#undef TL_BRANCH_CASE
-    TL_CHECK_LAUNCH("tl_branch_norm_add");
-    return 0;
-}
-
 // ---- residual add + RMSNorm ----------------------------------------------------------------
 // Without `rows`: x[r] += residual[r] (written back, float), out[r] = x[r] * rstd * w.
 // With `rows`:    out[r] = norm(x[rows[r]] + residual[rows[r]]); x is left as it is.
@@ -293,6 +233,149 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict
             tl_store4(orow + 4 * c4, o);
         }
     }
+}
+
+// ---- a normed branch added to the stream, and the next norm -------------------------------------
+// A residual branch whose output y is RMS-normed before it joins the stream:
+//   x[r] += mult * y[r] / sqrt(mean(y[r]^2) + eps_b) * wb
+// and, with w, the norm that reads the stream next, out[r] = x[r] / sqrt(mean(x[r]^2) + eps) * w, in the
+// same pass.  With `rows`: out only, for x[rows[r]] and y[rows[r]]; x is left as it is.  Float sums.
+template <typename O, bool HAS_ROWS>
+__global__ __launch_bounds__(1024) void branch_norm_add_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                               const float* __restrict__ wb, float mult, float eps_b,
+                                                               const float* __restrict__ w, float eps, O* __restrict__ out,
+                                                               const int32_t* __restrict__ rows, int H) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t src = HAS_ROWS ? (size_t)rows[r] : (size_t)r;
+    float* xr = x + src * H;
+    const float* yr = y + src * H;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) ss += yr[c] * yr[c];
+    ss = tl_block_sum(ss, red);
+    const float f = mult / sqrtf(ss / (float)H + eps_b);
+    float sx = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        const float v = xr[c] + yr[c] * f * wb[c];
+        if (!HAS_ROWS) xr[c] = v;
+        sx += v * v;
+    }
+    if (!w) return;
+    sx = tl_block_sum(sx, red);
+    const float rstd = 1.0f / sqrtf(sx / (float)H + eps);
+    O* orow = out + (size_t)r * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        const float v = HAS_ROWS ? xr[c] + yr[c] * f * wb[c] : xr[c];
+        orow[c] = tl_from_float<O>(v * rstd * w[c]);
+    }
+}
+
+// The same for H a multiple of 4 and at most 16384: one pass over memory, 16-byte accesses, the rows of y and of
+// the new x kept in registers between the sums and the scalings.
+template <typename O, bool HAS_ROWS>
+__global__ __launch_bounds__(1024) void branch_norm_add_vec_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                                   const float* __restrict__ wb, float mult, float eps_b,
+                                                                   const float* __restrict__ w, float eps, O* __restrict__ out,
+                                                                   const int32_t* __restrict__ rows, int H) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t src = HAS_ROWS ? (size_t)rows[r] : (size_t)r;
+    float* xr = x + src * H;
+    const float* yr = y + src * H;
+    const int n4 = H >> 2;
+    float4 v[NORM_VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NORM_VPT; ++i) {
+        const int c4 = threadIdx.x + i * blockDim.x;
+        if (c4 < n4) {
+            v[i] = tl_load4(yr + 4 * c4);
+            ss += v[i].x * v[i].x;
+            ss += v[i].y * v[i].y;
+            ss += v[i].z * v[i].z;
+            ss += v[i].w * v[i].w;
+        }
+    }
+    ss = tl_block_sum(ss, red);
+    const float f = mult / sqrtf(ss / (float)H + eps_b);
+    float sx = 0.f;
+#pragma unroll
+    for (int i = 0; i < NORM_VPT; ++i) {
+        const int c4 = threadIdx.x + i * blockDim.x;
+        if (c4 < n4) {
+            const float4 a = tl_load4(xr + 4 * c4), g = tl_load4(wb + 4 * c4);
+            float4 n;
+            n.x = a.x + v[i].x * f * g.x;
+            n.y = a.y + v[i].y * f * g.y;
+            n.z = a.z + v[i].z * f * g.z;
+            n.w = a.w + v[i].w * f * g.w;
+            if (!HAS_ROWS) tl_store4(xr + 4 * c4, n);
+            v[i] = n;
+            sx += n.x * n.x;
+            sx += n.y * n.y;
+            sx += n.z * n.z;
+            sx += n.w * n.w;
+        }
+    }
+    if (!w) return;
+    sx = tl_block_sum(sx, red);
+    const float rstd = 1.0f / sqrtf(sx / (float)H + eps);
+    O* orow = out + (size_t)r * H;
+#pragma unroll
+    for (int i = 0; i < NORM_VPT; ++i) {
+        const int c4 = threadIdx.x + i * blockDim.x;
+        if (c4 < n4) {
+            const float4 g = tl_load4(w + 4 * c4);
+            float4 o;
+            o.x = v[i].x * rstd * g.x;
+            o.y = v[i].y * rstd * g.y;
+            o.z = v[i].z * rstd * g.z;
+            o.w = v[i].w * rstd * g.w;
+            tl_store4(orow + 4 * c4, o);
+        }
+    }
+}
+
+extern "C" int tl_branch_norm_add(float* x, const float* y, const float* wb, float mult, float eps_b, const float* w, float eps,
+                                  void* out, int out_dtype, const int32_t* rows, int n_rows, int H, hipStream_t stream) {
+    TL_CHECK_ARG(n_rows >= 0 && H > 0 && eps >= 0.f && eps_b >= 0.f, "tl_branch_norm_add: bad sizes rows=%d H=%d", n_rows, H);
+    TL_CHECK_ARG((w == nullptr) == (out == nullptr) && (rows == nullptr || w != nullptr), "tl_branch_norm_add: a norm needs its output, and rows a norm");
+    if (n_rows == 0) return 0;
+    const bool vec = H % 4 == 0 && H <= 1024 * 4 * NORM_VPT;
+    int threads = (((vec ? H / 4 : H) + 63) / 64) * 64;
+    if (threads > 1024) threads = 1024;
+    dim3 grid(n_rows), block(threads);
+#define TL_BRANCH_VEC(OT)                                                                                                            \
+    do {                                                                                                                             \
+        if (rows)                                                                                                                    \
+            hipLaunchKernelGGL((branch_norm_add_vec_kernel<OT, true>), grid, block, 0, stream, x, y, wb, mult, eps_b, w, eps, (OT*)out, \
+                               rows, H);                                                                                             \
+        else                                                                                                                         \
+            hipLaunchKernelGGL((branch_norm_add_vec_kernel<OT, false>), grid, block, 0, stream, x, y, wb, mult, eps_b, w, eps,          \
+                               (OT*)out, rows, H);                                                                                   \
+    } while (0)
+    if (vec && (out_dtype == TL_BF16 || out_dtype == TL_F32)) {
+        if (out_dtype == TL_BF16) TL_BRANCH_VEC(bf16_t);
+        else TL_BRANCH_VEC(float);
+        TL_CHECK_LAUNCH("tl_branch_norm_add");
+        return 0;
+    }
+#undef TL_BRANCH_VEC
+#define TL_BRANCH_CASE(OT)                                                                                                       \
+    do {                                                                                                                         \
+        if (rows)                                                                                                                \
+            hipLaunchKernelGGL((branch_norm_add_kernel<OT, true>), grid, block, 0, stream, x, y, wb, mult, eps_b, w, eps, (OT*)out, \
+                               rows, H);                                                                                         \
+        else                                                                                                                     \
+            hipLaunchKernelGGL((branch_norm_add_kernel<OT, false>), grid, block, 0, stream, x, y, wb, mult, eps_b, w, eps,          \
+                               (OT*)out, rows, H);                                                                               \
+    } while (0)
+    if (out_dtype == TL_BF16) TL_BRANCH_CASE(bf16_t);
+    else if (out_dtype == TL_F32) TL_BRANCH_CASE(float);
+    else return tl_fail("tl_branch_norm_add: unknown dtype %d", out_dtype);
+#undef TL_BRANCH_CASE
+    TL_CHECK_LAUNCH("tl_branch_norm_add");
+    return 0;
 }
 
 template <typename R, typename O>
