@@ -220,11 +220,12 @@ extern "C" int tl_gated_scan(const float* gr, const float* gi, int ldg, const fl
 // ---- convolution, rotation and cache write of an attention layer's projections in one pass ------------------
 // proj float [T, >= C] holds a token's projected queries, keys and values side by side (biases added):
 // Hq query heads of d, Gk key heads of d, Gv value heads of dv; C = (Hq + Gk) d + Gv dv.  Each channel
-// goes through its short causal convolution (taps [C, K], the kept inputs as in tl_causal_conv), then
+// goes through its short causal convolution (taps [K, C], a tap's weights for all channels in a row, the last tap
+// the current token's; the kept inputs as in tl_causal_conv), then
 //   * queries and keys: the first `rot` dimensions of every head are turned in neighbouring pairs,
 //     (u, v) at dimensions (2i, 2i + 1) -> (u c - v s, v c + u s) with c = mag cos(pos f_i), s = mag
 //     sin(pos f_i), the angle in float (freq null or rot 0: no rotation);
-//   * queries are written to q_out [T, Hq, D] (columns d .. D - 1 are left as they are);
+//   * queries are written to q_out [T, Hq, D], zeros in columns d .. D - 1;
 //   * keys go into k_cache at the token's slot ([pages, page, Gk, D]) and values into v_cache with a
 //     page's tokens innermost ([pages, Gv v_rep, D, page]), every value head v_rep times in a row (a
 //     key head 2g + m then finds the values of g at its own index); padding columns are not written.
@@ -241,6 +242,11 @@ __global__ __launch_bounds__(256) void conv_rotate_store_kernel(
     int v_rep, int page, int C, int K, int shift) {
     const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
     const bool live = c < C;
+    if (D > d) {                                    // the queries' padding columns: zeros
+        const int w = D - d;
+        for (int idx = blockIdx.y * blockDim.x + threadIdx.x; idx < Hq * w; idx += blockDim.x * gridDim.y)
+            q_out[((size_t)t * Hq + idx / w) * D + d + idx % w] = tl_from_float<O>(0.f);
+    }
     const int s = seq_of_token[t];
     const int r0 = q_start[s];
     float* old = kept + (size_t)state_slots[s] * state_stride;
@@ -265,10 +271,10 @@ __global__ __launch_bounds__(256) void conv_rotate_store_kernel(
             const int r = t - (K - 1) + j;
             const float v = r >= r0 ? proj[(size_t)r * ldp + c] : old[(size_t)(r - r0 + K - 1) * C + c];
             seen[j] = v;
-            mine += taps[(size_t)c * K + j] * v;
+            mine += taps[(size_t)j * C + c] * v;
             if (turns) {
                 const float v2 = r >= r0 ? proj[(size_t)r * ldp + c2] : old[(size_t)(r - r0 + K - 1) * C + c2];
-                other += taps[(size_t)c2 * K + j] * v2;
+                other += taps[(size_t)j * C + c2] * v2;
             }
         }
     }
@@ -326,6 +332,11 @@ __global__ __launch_bounds__(256) void conv_rotate_store_vec_kernel(
     int v_rep, int page, int C, int K, int shift) {
     __shared__ float cs_s[128], sn_s[128];          // one cosine and sine per rotated pair of the token, times mag
     const int t = blockIdx.x;
+    if (D > d) {                                    // the queries' padding columns: zeros
+        const int w = D - d;
+        for (int idx = blockIdx.y * blockDim.x + threadIdx.x; idx < Hq * w; idx += blockDim.x * gridDim.y)
+            q_out[((size_t)t * Hq + idx / w) * D + d + idx % w] = tl_from_float<O>(0.f);
+    }
     if (freq != nullptr) {
         const float p = (float)pos[t];
         for (int i = threadIdx.x; i < (rot >> 1); i += blockDim.x) {
@@ -342,16 +353,16 @@ __global__ __launch_bounds__(256) void conv_rotate_store_vec_kernel(
     const int slot = slots ? slots[t] : -1;
     const int qk = (Hq + Gk) * d;
   for (int c = 4 * (blockIdx.y * blockDim.x + threadIdx.x); c < C; c += 4 * blockDim.x * gridDim.y) {
-    const float* tp = taps + (size_t)c * K;             // the four channels' taps, 4 K floats in a row
     float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int j = 0; j < K; ++j) {
         const int r = t - (K - 1) + j;
         const float4 v = r >= r0 ? *reinterpret_cast<const float4*>(proj + (size_t)r * ldp + c)
                                  : *reinterpret_cast<const float4*>(old + (size_t)(r - r0 + K - 1) * C + c);
-        y.x += tp[j] * v.x;
-        y.y += tp[K + j] * v.y;
-        y.z += tp[2 * K + j] * v.z;
-        y.w += tp[3 * K + j] * v.w;
+        const float4 w = *reinterpret_cast<const float4*>(taps + (size_t)j * C + c);
+        y.x += w.x * v.x;
+        y.y += w.y * v.y;
+        y.z += w.z * v.z;
+        y.w += w.w * v.w;
         if (shift && j > 0) *reinterpret_cast<float4*>(old + (size_t)(j - 1) * C + c) = v;
     }
     if (c < qk) {
@@ -408,7 +419,7 @@ extern "C" int tl_conv_rotate_store(const float* proj, int ldp, const float* tap
     if (T == 0 || S == 0) return 0;
     if (rot == 0) freq = nullptr;
     const int shift = update == 2 ? 1 : 0;
-    const bool vec = rot <= 256 && d % 4 == 0 && dv % 4 == 0 && D % 4 == 0 && ldp % 4 == 0 && (uintptr_t)proj % 16 == 0 && (uintptr_t)kept % 16 == 0 &&
+    const bool vec = rot <= 256 && C % 4 == 0 && (uintptr_t)taps % 16 == 0 && d % 4 == 0 && dv % 4 == 0 && D % 4 == 0 && ldp % 4 == 0 && (uintptr_t)proj % 16 == 0 && (uintptr_t)kept % 16 == 0 &&
                      state_stride % 4 == 0 && (uintptr_t)q_out % 16 == 0 && (uintptr_t)k_cache % 16 == 0;
     if (vec && (dtype == TL_F32 || dtype == TL_BF16)) {
         dim3 vblock(256), vgrid(T, tl_ceil_div(C, 1024));

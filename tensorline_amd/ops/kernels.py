@@ -1444,7 +1444,8 @@ def conv_rotate_store(proj: torch.Tensor, taps: torch.Tensor, ctx, state: torch.
                       out_dtype: torch.dtype) -> torch.Tensor:
     """What lies between the fused q/k/v projection of an attention layer with short convolutions and attention, in
     one pass per token.  ``proj`` float32 [T, >= C], C = (heads + k_heads) * dim + v_heads * vdim, biases added
-    (columns beyond C are not looked at).  Every channel goes through its causal convolution (``taps`` float32 [C, K];
+    (columns beyond C are not looked at).  Every channel goes through its causal convolution (``taps`` float32 [K, C],
+    a tap's weights for all channels in a row, the last tap the current token's;
     the inputs ahead of the step's first row are the K - 1 rows kept at ``state[slot, offset : offset + (K - 1) C]``,
     renewed afterwards); queries and keys are then turned in neighbouring pairs (2i, 2i + 1) over their first
     ``2 * len(freq)`` dimensions by the angle ``pos * freq[i]``, cosine and sine times ``mag`` (``freq`` None: no
@@ -1455,10 +1456,10 @@ def conv_rotate_store(proj: torch.Tensor, taps: torch.Tensor, ctx, state: torch.
     _on_gpu(proj, taps, state, freq, k_cache, v_cache, slots)
     T = proj.shape[0]
     C = (heads + k_heads) * dim + v_heads * vdim
-    K = taps.shape[1]
+    K = taps.shape[0]
     _check(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= C,
            "conv_rotate_store: the projection must be float32 [T, >= C]")
-    _check(taps.dim() == 2 and taps.shape[0] == C and 1 <= K <= CONV_MAX_TAPS, f"conv_rotate_store: taps must be [{C}, up to {CONV_MAX_TAPS}]")
+    _check(taps.dim() == 2 and taps.shape[1] == C and 1 <= K <= CONV_MAX_TAPS, f"conv_rotate_store: taps must be [up to {CONV_MAX_TAPS}, {C}]")
     _f32(taps, "conv_rotate_store taps")
     _check(state.dtype == torch.float32 and offset + (K - 1) * C <= state.shape[1], "conv_rotate_store: the kept inputs do not fit the state")
     rot = 0
@@ -1476,7 +1477,7 @@ def conv_rotate_store(proj: torch.Tensor, taps: torch.Tensor, ctx, state: torch.
     else:
         _check(v_heads == 0, "conv_rotate_store: values come with keys")
     _i32(ctx.pos, "pos", T)
-    q = (torch.empty if head_size == dim else torch.zeros)(T, heads * head_size, dtype=out_dtype, device=proj.device)
+    q = torch.empty(T, heads * head_size, dtype=out_dtype, device=proj.device)
     kept, stride = _state_ptr(state, offset)
     one_launch = ctx.facts.decode_only and T == ctx.num_seqs and (rot == 0 or dim % 2 == 0)
     _call("tl_conv_rotate_store", _ptr(proj), proj.stride(0) if T > 1 else max(C, proj.stride(0)), _ptr(taps), kept,

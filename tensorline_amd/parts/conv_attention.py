@@ -109,7 +109,7 @@ class _ConvAttention(Part):
             if q.bias is not None:
                 q.bias = q.bias.index_select(0, order).contiguous()
             taps[0] = taps[0].index_select(0, order)
-        self.taps = torch.cat(taps, dim=0).contiguous()
+        self.taps = torch.cat(taps, dim=0).t().contiguous()        # [taps, channels]: a tap's weights in a row
         parts = list(self._projs)
         D = self.kernel_dim
         if self._gate is not None:

@@ -172,7 +172,7 @@ def test_convolution_rotation_and_cache_write_in_one_pass(case):
     planes = cache.storage(0)
     keys, values = (planes["k"], planes["v"]) if Gk else (None, None)
     ctx, views = _step_context(cache, runner, [("old", 0, 9)])                # leaves its inputs in slot 0 ...
-    kernels.conv_rotate_store(torch.randn(9, C, device=DEV), taps.to(DEV), ctx, state, 5, freq.to(DEV) if rot else None, mag, keys,
+    kernels.conv_rotate_store(torch.randn(9, C, device=DEV), taps.t().contiguous().to(DEV), ctx, state, 5, freq.to(DEV) if rot else None, mag, keys,
                               values, views[0].slots if Gk else None, Hq, Gk, d, Gv, dv, D, rep, torch.float32)
     cache.release("old")                                                      # ... which "a" gets: the test zeroes it as the manager does
     state.zero_()
@@ -181,7 +181,7 @@ def test_convolution_rotation_and_cache_write_in_one_pass(case):
     for step in ([("a", 1), ("b", 5)], [("a", 2)], [("a", 1), ("b", 1)], [("b", 2), ("a", 19)], [("a", 1)], [("a", 6), ("b", 4)]):
         ctx, views = _step_context(cache, runner, [(r, at[r], n) for r, n in step])
         x = torch.cat([xs[r][at[r]:at[r] + n] for r, n in step]).to(DEV)
-        got = kernels.conv_rotate_store(x, taps.to(DEV), ctx, state, 5, freq.to(DEV) if rot else None, mag, keys, values,
+        got = kernels.conv_rotate_store(x, taps.t().contiguous().to(DEV), ctx, state, 5, freq.to(DEV) if rot else None, mag, keys, values,
                                         views[0].slots if Gk else None, Hq, Gk, d, Gv, dv, D, rep, torch.float32).cpu()
         got = got.view(-1, Hq, D)
         row = 0
