@@ -223,8 +223,8 @@ def test_normed_branch_joins_the_stream_in_the_next_norm():
         torch.manual_seed(H)
         x, y = torch.randn(7, H), torch.randn(7, H) * 3
         wb, wn = torch.randn(H), torch.randn(H)
-        x2 = x + 0.7 * P.rms_norm(y, wb, 1e-5)
-        branch = kernels.NormedBranch(y.to(DEV), wb.to(DEV), 1e-5, 0.7)
+        x2 = x + 0.45 * P.rms_norm(y, wb, 2e-5)
+        branch = kernels.NormedBranch(y.to(DEV), wb.to(DEV), 2e-5, 0.45)
         xd = x.to(DEV)
         rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
         picked = kernels.add_rmsnorm(xd, branch, wn.to(DEV), 1e-6, torch.float32, rows=rows).cpu()
