@@ -5,8 +5,8 @@ their projection, over the framework's paged cache, in two kinds:
   (YaRN's frequencies) over the first ``rot.dims`` dimensions of a head, an optional window, an optional
   output gate ``sigmoid(W_g h)`` on the concatenated heads, biases on q/k/v (``bias``) and on the output
   projection (``out_bias``);
-* ``differential_attention``: every head has two maps (queries and keys laid out head by head as [map 1,
-  map 2]) over the same values; ``o = a1 - lambda a2`` with ``lambda = exp(lq1 . lk1) - exp(lq2 . lk2) +
+* ``differential_attention``: every head has two maps (a head's query rows, and a key head's rows, are those of map 1
+  followed by those of map 2) over the same values; ``o = a1 - lambda a2`` with ``lambda = exp(lq1 . lk1) - exp(lq2 . lk2) +
   diff``, one number per layer, then ``o / rms(o) * (1 - diff)`` per head.  No rotation.
 
 Both: tensors ``q``, ``k``, ``v`` (``.b`` biases, ``.conv`` taps [channels, taps]), ``o``; ``kv_proj`` False
