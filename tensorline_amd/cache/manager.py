@@ -52,6 +52,10 @@ class CacheGroup:
     def window(self) -> int:
         return self.need.window
 
+    @property
+    def trims(self) -> bool:
+        return self.need.trims
+
 
 @dataclass
 class _Request:
@@ -99,12 +103,14 @@ class CacheManager:
             self.groups[g].entries.append(i)
             self.group_of_entry[i] = g
             self.storage_entry[i] = i
-        self._windowed = any(g.window > 0 for g in self.groups)
+        self._windowed = any(g.trims for g in self.groups)
         self._serial = 0
         # an entry that reads a windowed entry's cache with a wider view would see freed pages
         for i, e in enumerate(schedule):
             if e.cache_from is not None and cache_needs[i] is not None:
                 src_w, my_w = cache_needs[e.cache_from].window, cache_needs[i].window
+                if cache_needs[e.cache_from].chunk != cache_needs[i].chunk or cache_needs[e.cache_from].keep_first < cache_needs[i].keep_first:
+                    raise ValueError(f"schedule entry {i} sees other tokens than the cache of entry {e.cache_from} keeps")
                 if src_w > 0 and (my_w == 0 or my_w > src_w):
                     raise ValueError(f"schedule entry {i} looks further back than the cache of entry {e.cache_from} keeps")
 
@@ -117,7 +123,7 @@ class CacheManager:
 
         # prefix sharing: only where one page id means the same tokens for every layer and no
         # mixer carries state that pages do not hold
-        self.prefix_caching = bool(prefix_caching) and len(self.groups) == 1 and self.groups[0].window == 0 \
+        self.prefix_caching = bool(prefix_caching) and len(self.groups) == 1 and not self.groups[0].trims \
             and not self.has_state
         if self.prefix_caching:
             self.groups[0].allocator.share_prefixes = True
@@ -168,8 +174,10 @@ class CacheManager:
         """Could a request of ``tokens`` tokens be held if it were alone?  A windowed group needs
         pages for its window plus one step's portion only."""
         for g in self.groups:
-            if g.window > 0:
-                span = min(tokens, g.window + step_tokens + self.page_size)
+            if g.trims:
+                reach = min(r for r in (g.window, g.need.chunk) if r > 0)
+                kept = -(-g.need.keep_first // self.page_size) * self.page_size
+                span = min(tokens, reach + kept + step_tokens + self.page_size)
             else:
                 span = tokens
             if self.pages_for(span) > self.num_blocks:
@@ -249,14 +257,15 @@ class CacheManager:
         req = self._requests[rid]
         given = 0
         for gi, g in enumerate(self.groups):
-            if g.window <= 0:
+            if not g.trims:
                 continue
-            first_needed = computed - g.window + 1
+            first_needed = g.need.first_needed(computed)
             if first_needed <= 0:
                 continue
             upto_page = min(first_needed // self.page_size, len(req.tables[gi]))
+            kept_pages = -(-g.need.keep_first // self.page_size)     # the first tokens stay for good
             back = []
-            for lp in range(req.trimmed[gi], upto_page):
+            for lp in range(max(req.trimmed[gi], kept_pages), upto_page):
                 if req.tables[gi][lp] >= 0:
                     back.append(req.tables[gi][lp])
                     req.tables[gi][lp] = -1

@@ -5,3 +5,4 @@ from tensorline_amd.config.registry import (  # noqa: F401
 from tensorline_amd.config.samovik_config import SamovikConfig  # noqa: F401
 from tensorline_amd.config.tumitar_config import TumitarConfig  # noqa: F401
 from tensorline_amd.config.zeganex_config import ZeganexConfig  # noqa: F401
+from tensorline_amd.config.kabulix_config import KabulixConfig  # noqa: F401

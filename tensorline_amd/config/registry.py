@@ -78,3 +78,4 @@ def _ensure_builtin() -> None:
     import tensorline_amd.models.samovik  # noqa: F401
     import tensorline_amd.models.tumitar  # noqa: F401
     import tensorline_amd.models.zeganex  # noqa: F401
+    import tensorline_amd.models.kabulix  # noqa: F401

@@ -10,18 +10,20 @@ void tl_attention_generic_bf16(const AgLaunch& a);
 // and a second kernel merges them: for steps of few tokens with long contexts, which would
 // otherwise be walked by one work-group per sequence and key/value head.  nsplit * split_keys must
 // cover the longest context; ws holds T * nq * nsplit * (d + 2) floats.  sink != 0: one is added to the
-// softmax's denominator (a key of score 0 that has no value).
+// softmax's denominator (a key of score 0 that has no value).  window, chunk, keep_first: which keys a
+// token sees (TlMask).
 extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                     const int32_t* tables, int NB, const int32_t* q_start, const int32_t* pos,
                                     void* out, int out_stride, int dtype, int T, int S, int max_query_len, int nq, int nkv,
                                     int d, int bs, int window, float scale, int nsplit, int split_keys, float* ws,
-                                    int sink, hipStream_t stream) {
+                                    int sink, int keep_first, int chunk, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && d > 0 && bs > 0 && NB > 0,
                  "tl_attention_generic: bad sizes T=%d S=%d nq=%d nkv=%d d=%d page=%d NB=%d", T, S, nq, nkv, d, bs, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_generic: %d query heads are not a multiple of %d key/value heads", nq, nkv);
     TL_CHECK_ARG(d <= 256 && d % 16 == 0, "tl_attention_generic: head size %d must be a multiple of 16 and at most 256", d);
     TL_CHECK_ARG(nkv <= 65535, "tl_attention_generic: too many key/value heads %d", nkv);
     TL_CHECK_ARG(q_stride >= nq * d && out_stride >= nq * d, "tl_attention_generic: row strides too small");
+    TL_CHECK_ARG(window >= 0 && keep_first >= 0 && chunk >= 0, "tl_attention_generic: negative window, chunk or kept first keys");
     TL_CHECK_ARG(max_query_len >= 1 || T == 0, "tl_attention_generic: max_query_len %d", max_query_len);
     if (T == 0 || S == 0) return 0;
     const int G = nq / nkv;
@@ -51,7 +53,7 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
     a.q = q; a.k_cache = k_cache; a.v_cache = v_cache; a.tables = tables; a.q_start = q_start; a.pos = pos; a.out = out;
     a.ws_o = ws_o; a.ws_ml = ws_ml; a.q_stride = q_stride; a.NB = NB; a.out_stride = out_stride; a.T = T;
     a.tiles_per_seq = tiles_per_seq; a.QT = QT; a.GC = GC; a.nq = nq; a.nkv = nkv; a.d = d; a.bs = bs; a.bs_shift = bs_shift;
-    a.window = window; a.nsplit = nsplit; a.split_keys = split_keys; a.scale = scale; a.keys_over_waves = keys_over_waves;
+    a.mask = TlMask{window, chunk, keep_first}; a.nsplit = nsplit; a.split_keys = split_keys; a.scale = scale; a.keys_over_waves = keys_over_waves;
     a.grid = dim3((unsigned)groups, nkv, chunks * nsplit);
     a.smem = smem; a.stream = stream; a.sink = sink;
     if (dtype == TL_F32)

@@ -4,8 +4,9 @@
 // out, no reduced precision anywhere): this is the attention of the true 32-bit path, and of
 // bfloat16 shapes the bfloat16 matrix-core kernel does not take.
 //
-// A token at position p of sequence s attends to keys [lo, p] of that sequence, lo = 0 or
-// p - window + 1 for a windowed layer, found through the sequence's row of the page table.  The
+// A token at position p of sequence s attends to keys [lo, p] of that sequence, lo = 0, p - window + 1
+// for a windowed layer or the start of p's chunk for a chunked one, and to the first keys a layer keeps
+// in sight for good (TlMask), found through the sequence's row of the page table.  The
 // keys of the step's own tokens are already in the cache when this runs.  k_cache is
 // [pages, page, nkv, d]; v_cache is [pages, nkv, d, page] (reference: tensorline/paged_attn.py:25-58,
 // tensorline/paged.py:233-238).
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
     T* __restrict__ out, int out_stride, int tiles_per_seq, int QT, int GC, int nq, int nkv, int bs, int bs_shift,
-    int window, float scale, int nsplit, int split_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml, int sink) {
+    TlMask mask, float scale, int nsplit, int split_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml, int sink) {
     constexpr int d = DB * 16;
     constexpr int KT = AG_KT(d, KW);
     extern __shared__ float smem[];
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
         int p = -1, lo = 0;
         if (i < nt && g < gc) {
             p = pos[t_first + i];
-            lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+            lo = tl_mask_lo(mask, p);
         }
         row_pos[tid] = p;
         row_lo[tid] = lo;
@@ -265,20 +266,33 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     // With split keys this work-group walks the tiles of split sp only: keys [sp * split_keys,
     // (sp + 1) * split_keys), a multiple of KT at absolute positions, so that the same keys are summed
     // together whatever the context length and the number of splits of the launch.
-    int k_first = (k_lo / KT) * KT, k_end = k_hi;
+    // Where the rows' ranges start beyond the kept first keys (k_lo > 0 then holds for every row), the
+    // tiles of those keys, [0, head_end), are walked first and the tiles in between are left out.
+    const int k_main = (k_lo / KT) * KT;
+    int head_end = 0;
+    if (mask.first > 0 && k_main > 0) {
+        head_end = ((mask.first + KT - 1) / KT) * KT;
+        head_end = (head_end < k_main) ? head_end : k_main;
+    }
+    int k_first = head_end > 0 ? 0 : k_main, k_end = k_hi;
     if (nsplit > 1) {
-        k_first = (k_first > sp * split_keys) ? k_first : sp * split_keys;
+        const int s_lo = sp * split_keys;
+        if (s_lo > k_first) k_first = (s_lo < head_end || s_lo > k_main) ? s_lo : k_main;
         k_end = (k_end < (sp + 1) * split_keys) ? k_end : (sp + 1) * split_keys;
     }
+    auto tile_after = [&](int k0) {
+        const int n = k0 + KT;
+        return (n >= head_end && n < k_main) ? k_main : n;
+    };
     constexpr int key_blocks = KT / 16;
     if (k_first < k_end) fetch(k_first);
-    for (int k0 = k_first; k0 < k_end; k0 += KT) {
+    for (int k0 = k_first; k0 < k_end; k0 = tile_after(k0)) {
         to_lds(k0);
         __syncthreads();
-        if (k0 + KT < k_end) fetch(k0 + KT);
+        if (tile_after(k0) < k_end) fetch(tile_after(k0));
 
         // a tile none of the wave's rows sees is skipped; KW: a wave without a key block of its own stands by
-        if (k0 < w_hi && k0 + KT > w_lo && (!KW || wave < key_blocks)) {
+        if (k0 < w_hi && (k0 + KT > w_lo || k0 < mask.first) && (!KW || wave < key_blocks)) {
             // ---- S = Q K^T: per block of 16 keys, 4 DB products; lane holds rows 4 lg + v, key li ----
             ag_f32x4 sblk[4];
 #pragma unroll
@@ -307,7 +321,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
                         continue;
                     }
                     const int key = k0 + (KW ? wave : jb) * 16 + li;
-                    const bool seen = (KW || jb < key_blocks) && my_pos[v] >= 0 && key <= my_pos[v] && key >= my_lo[v];
+                    const bool seen = (KW || jb < key_blocks) && my_pos[v] >= 0 && key <= my_pos[v] && !tl_mask_hides(mask, key, my_lo[v]);
                     sv[jb] = seen ? sblk[jb][v] : -INFINITY;
                     mx = fmaxf(mx, sv[jb]);
                 }
@@ -497,7 +511,8 @@ struct AgLaunch {
     const int32_t *tables, *q_start, *pos;
     void* out;
     float *ws_o, *ws_ml;
-    int q_stride, NB, out_stride, T, tiles_per_seq, QT, GC, nq, nkv, d, bs, bs_shift, window, nsplit, split_keys, sink;
+    int q_stride, NB, out_stride, T, tiles_per_seq, QT, GC, nq, nkv, d, bs, bs_shift, nsplit, split_keys, sink;
+    TlMask mask;
     float scale;
     bool keys_over_waves;
     dim3 grid;
@@ -515,7 +530,7 @@ static void ag_launch_all(const AgLaunch& a) {
 #define AG_LAUNCH_KW(DB, KWV)                                                                                         \
     hipLaunchKernelGGL((attn_generic_kernel<TT, DB, KWV>), a.grid, block, a.smem, a.stream, (const TT*)a.q,           \
                        a.q_stride, (const TT*)a.k_cache, (const TT*)a.v_cache, a.tables, a.NB, a.q_start, a.pos,      \
-                       (TT*)a.out, a.out_stride, a.tiles_per_seq, a.QT, a.GC, a.nq, a.nkv, a.bs, a.bs_shift, a.window, \
+                       (TT*)a.out, a.out_stride, a.tiles_per_seq, a.QT, a.GC, a.nq, a.nkv, a.bs, a.bs_shift, a.mask,   \
                        a.scale, a.nsplit, a.split_keys, a.ws_o, a.ws_ml, a.sink)
 #define AG_CASE(DB)                                                                                                   \
     case DB:                                                                                                          \

@@ -74,7 +74,7 @@ __device__ __forceinline__ float am_column_max(float v) {
 // no running maximum moved.
 template <int DC, int NT>
 __device__ __forceinline__ void am_block(const uint4* kf0, const uint4* kf1, const uint4* vf, const uint4 (*qf)[DC],
-                                         const int* p_col, const int* lo_col, int kb, int g, float scale2,
+                                         const int* p_col, const int* lo_col, int first, int kb, int g, float scale2,
                                          float* m_run, float* l_run, f32x4 (*acc)[DC * 2]) {
     constexpr int DB = DC * 2;
     const int key_base = kb + 8 * g;
@@ -97,7 +97,7 @@ __device__ __forceinline__ void am_block(const uint4* kf0, const uint4* kf1, con
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int key = key_base + i;
-                if (key > p_col[j] || key < lo_col[j]) sv[i] = -INFINITY;
+                if (key > p_col[j] || (key < lo_col[j] && key >= first)) sv[i] = -INFINITY;
             }
         }
         const float bmax = am_column_max(am_max3(am_max3(sv[0], sv[1], sv[2]), am_max3(sv[3], sv[4], sv[5]), am_max3(sv[6], sv[7], sv[7])));
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, float* __restrict__ ws_o,
-    float* __restrict__ ws_ml, int nq, int nkv, int bs, int bs_shift, int window, float scale, int nsplit,
+    float* __restrict__ ws_ml, int nq, int nkv, int bs, int bs_shift, TlMask mask, float scale, int nsplit,
     int split_blocks, const int32_t* __restrict__ seq_list, int skip_single, int sink) {
     constexpr int D = DC * 32;
     constexpr int DB = D / 16;
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
         head_col[j] = kvh * G + gh;
         has_col[j] = valid;
         p_col[j] = valid ? start + tok : AM_NO_COLUMN;
-        lo_col[j] = (valid && window > 0 && p_col[j] - window + 1 > 0) ? p_col[j] - window + 1 : 0;
+        lo_col[j] = valid ? tl_mask_lo(mask, p_col[j]) : 0;
         const bf16_t* qp = q + (size_t)row_col[j] * q_stride + (size_t)head_col[j] * D + g * 8;
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc)
@@ -194,18 +194,26 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     // ---- key range of the wave, in blocks of 32, and this split's share ----
     const int last_col = ((col0 + NT * 16 < ncols) ? col0 + NT * 16 : ncols) - 1;
     const int khi = start + last_col / G;                      // last key any column of the wave sees
-    int klo = 0;
-    if (window > 0) {
-        klo = start + col0 / G - window + 1;
-        if (klo < 0) klo = 0;
-    }
+    const int klo = tl_mask_lo(mask, start + col0 / G);       // of the first column: no column's is lower
     const int b_lo = klo >> 5, b_hi = khi >> 5;
-    int bb = b_lo, be = b_hi + 1;
+    // The blocks of the kept first keys, [0, hb), are walked ahead of the blocks from b_lo on where the
+    // two do not touch; this split's share of each: [ha, hb) and [bb, be).
+    int hb = 0;
+    if (mask.first > 0 && b_lo > 0) {
+        hb = (mask.first + 31) >> 5;
+        if (hb > b_lo) hb = b_lo;
+    }
+    int ha = 0, bb = b_lo, be = b_hi + 1;
     if (nsplit > 1) {
         if (sp * split_blocks > bb) bb = sp * split_blocks;
         if ((sp + 1) * split_blocks < be) be = (sp + 1) * split_blocks;
-        if (bb >= be) return;
+        if (sp * split_blocks > ha) ha = sp * split_blocks;
+        if ((sp + 1) * split_blocks < hb) hb = (sp + 1) * split_blocks;
     }
+    const int n_head = hb > ha ? hb - ha : 0;
+    const int n_blocks = n_head + (be > bb ? be - bb : 0);
+    if (n_blocks == 0) return;
+    const int b_first = n_head ? ha : bb, b_last = be > bb ? be - 1 : hb - 1;
 
     float m_run[NT], l_run[NT];
     f32x4 acc[NT][DB];
@@ -220,8 +228,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     // The page ids of the wave's keys, one per lane, when they are at most 64 (a split of a decode
     // step always is): a block's addresses then come from a lane exchange instead of a load from
     // memory that the loads of keys and values would have to wait for.
-    const int page_lo = am_page_index(bb << 5, bs, bs_shift);
-    const int last_key = ((be << 5) - 1 < khi) ? (be << 5) - 1 : khi;
+    const int page_lo = am_page_index(b_first << 5, bs, bs_shift);
+    const int last_key = ((b_last << 5) + 31 < khi) ? (b_last << 5) + 31 : khi;
     const int npages = am_page_index(last_key, bs, bs_shift) - page_lo + 1;
     const bool pages_in_lanes = npages <= 64;
     const int my_page = pages_in_lanes ? table[page_lo + (lane < npages ? lane : npages - 1)] : 0;
@@ -254,13 +262,15 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
         _Pragma("unroll") for (int db = 0; db < DB; ++db)                                                    \
             V[db] = *reinterpret_cast<const uint4*>(vp_ + (size_t)db * 16 * bs);                             \
     }
-    AM_LOAD_BLOCK(bb, kf0, kf1, vf)
-    for (int b = bb; b < be; ++b) {
+    AM_LOAD_BLOCK(b_first, kf0, kf1, vf)
+    for (int i = 0; i < n_blocks; ++i) {
+        const int b = i < n_head ? ha + i : bb + (i - n_head);
         const int kb = b << 5;
-        const int b_next = (b + 1 < be) ? b + 1 : b;
+        const int i_next = (i + 1 < n_blocks) ? i + 1 : i;
+        const int b_next = i_next < n_head ? ha + i_next : bb + (i_next - n_head);
         AM_LOAD_BLOCK(b_next, kn0, kn1, vn)
 
-        am_block<DC, NT>(kf0, kf1, vf, qf, p_col, lo_col, kb, g, scale2, m_run, l_run, acc);
+        am_block<DC, NT>(kf0, kf1, vf, qf, p_col, lo_col, mask.first, kb, g, scale2, m_run, l_run, acc);
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc) {
             kf0[dc] = kn0[dc];
@@ -313,8 +323,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
 // fragments are dead before value fragments are read: few registers are live at once.
 template <int DC, int NT>
 __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, int kx, int vx, int half,
-                                             const uint4 (*qf)[DC], const int* p_col, const int* lo_col, int kb, int c,
-                                             int g, float scale2, float* m_run, float* l_run, f32x4 (*acc)[DC * 2]) {
+                                             const uint4 (*qf)[DC], const int* p_col, const int* lo_col, int first, int kb,
+                                             int c, int g, float scale2, float* m_run, float* l_run, f32x4 (*acc)[DC * 2]) {
     constexpr int DB = DC * 2;
     constexpr int UPK = DC * 4;
     const int key_base = kb + 8 * g;
@@ -345,7 +355,7 @@ __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, i
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int key = key_base + i;
-                if (key > p_col[j] || key < lo_col[j]) sv[i] = -INFINITY;
+                if (key > p_col[j] || (key < lo_col[j] && key >= first)) sv[i] = -INFINITY;
             }
         }
         const float bmax = am_column_max(am_max3(am_max3(sv[0], sv[1], sv[2]), am_max3(sv[3], sv[4], sv[5]), am_max3(sv[6], sv[7], sv[7])));
@@ -398,8 +408,8 @@ __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, i
 // fragments of the first 32 keys while the softmax is computed.
 template <int DC>
 __device__ __forceinline__ void am_tile_lds(const uint4* kt, const uint4* vt, int kx, int vx, const uint4* qf,
-                                            int p_col, int lo_col, int kb, int c, int g, float scale2, float& m_run,
-                                            float& l_run, f32x4* acc) {
+                                            int p_col, int lo_col, int first, int kb, int c, int g, float scale2,
+                                            float& m_run, float& l_run, f32x4* acc) {
     constexpr int DB = DC * 2;
     constexpr int UPK = DC * 4;
     f32x4 st[4];
@@ -451,7 +461,7 @@ __device__ __forceinline__ void am_tile_lds(const uint4* kt, const uint4* vt, in
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int key = kb + 32 * h + 8 * g + i;
-                if (key > p_col || key < lo_col) sv[8 * h + i] = -INFINITY;
+                if (key > p_col || (key < lo_col && key >= first)) sv[8 * h + i] = -INFINITY;
             }
     }
     float bmax = am_max3(am_max3(am_max3(sv[0], sv[1], sv[2]), am_max3(sv[3], sv[4], sv[5]), sv[6]),
@@ -554,7 +564,7 @@ __global__ __launch_bounds__(CH * WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int S, int nq, int nkv, int bs,
-    int bs_shift, int window, float scale, int skip_single, int sink) {
+    int bs_shift, TlMask mask, float scale, int skip_single, int sink) {
     constexpr int THREADS = CH * WAVES * 64;
     constexpr int WCOLS = NT * 16;                       // columns of a wave; WAVES * WCOLS = 128 per work-group
     constexpr int D = DC * 32;
@@ -636,21 +646,23 @@ __global__ __launch_bounds__(CH * WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     // key range of the work-group and of this wave
     const int wg_last = ((wg_col0 + 128 < ncols) ? wg_col0 + 128 : ncols) - 1;
     const int khi = start + wg_last / G;
-    int klo = 0;
-    if (window > 0) {
-        klo = start + wg_col0 / G - window + 1;
-        if (klo < 0) klo = 0;
-    }
+    const int klo = tl_mask_lo(mask, start + wg_col0 / G);   // of the first column: no column's is lower
     const int t_lo = klo / AT_KEYS, t_hi = khi / AT_KEYS;
+    // The tiles of the kept first keys, [0, t_head), are walked ahead of the tiles from t_lo on where the
+    // two do not touch: walk step i takes tile i below t_head and tile t_lo + i - t_head from there on.
+    int t_head = 0;
+    if (mask.first > 0 && t_lo > 0) {
+        t_head = (mask.first + AT_KEYS - 1) / AT_KEYS;
+        if (t_head > t_lo) t_head = t_lo;
+    }
+    const int t_shift = t_lo - t_head, n_tiles = t_head + t_hi - t_lo + 1;
+#define AT_TILE_AT(I) ((I) < t_head ? (I) : (I) + t_shift)
+    const int first_key = mask.first;
     int wk_lo = 1, wk_hi = 0;                 // empty for a wave without columns
     if (wave_active) {
         const int w_last = ((col0 + WCOLS < ncols) ? col0 + WCOLS : ncols) - 1;
         wk_hi = start + w_last / G;
-        wk_lo = 0;
-        if (window > 0) {
-            wk_lo = start + col0 / G - window + 1;
-            if (wk_lo < 0) wk_lo = 0;
-        }
+        wk_lo = tl_mask_lo(mask, start + col0 / G);
     }
     // page ids into LDS
     {
@@ -672,7 +684,7 @@ __global__ __launch_bounds__(CH * WAVES * 64, 32 / WAVES) void attn_tile_kernel(
         head_col[j] = kvh * G + gh;
         has_col[j] = valid;
         p_col[j] = valid ? start + tok : AM_NO_COLUMN;
-        lo_col[j] = (valid && window > 0 && p_col[j] - window + 1 > 0) ? p_col[j] - window + 1 : 0;
+        lo_col[j] = valid ? tl_mask_lo(mask, p_col[j]) : 0;
         const bf16_t* qp = q + (size_t)row_col[j] * q_stride + (size_t)head_col[j] * D + g * 8;
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc)
@@ -729,45 +741,50 @@ __global__ __launch_bounds__(CH * WAVES * 64, 32 / WAVES) void attn_tile_kernel(
         const uint4* vt = vs + cur * TILE;                                                                    \
         if (NT == 1 && (T) * AT_KEYS + 32 <= wk_hi && (T) * AT_KEYS + 31 >= wk_lo) {                          \
             /* both halves hold keys of the wave: the whole tile at once */                                   \
-            am_tile_lds<DC>(kt, vt, kx, vx, qf[0], p_col[0], lo_col[0], (T) * AT_KEYS, c, g, scale2, m_run[0], \
-                            l_run[0], acc[0]);                                                                \
+            am_tile_lds<DC>(kt, vt, kx, vx, qf[0], p_col[0], lo_col[0], first_key, (T) * AT_KEYS, c, g, scale2,   \
+                            m_run[0], l_run[0], acc[0]);                                                      \
         } else {                                                                                              \
             _Pragma("unroll") for (int half = 0; half < 2; ++half) {                                          \
                 const int kb = (T) * AT_KEYS + half * 32;                                                     \
-                if (kb > wk_hi || kb + 31 < wk_lo) continue; /* the same for the whole wave */                \
-                am_block_lds<DC, NT>(kt, vt, kx, vx, half, qf, p_col, lo_col, kb, c, g, scale2, m_run, l_run, acc); \
+                if (kb > wk_hi || (kb + 31 < wk_lo && kb >= first_key)) continue; /* the same for the whole wave */ \
+                am_block_lds<DC, NT>(kt, vt, kx, vx, half, qf, p_col, lo_col, first_key, kb, c, g, scale2, m_run, l_run, acc); \
             }                                                                                                 \
         }                                                                                                     \
     }
     int cur = 0;
     if (CH == 1) {
-        AT_FETCH(t_lo, 0)
+        AT_FETCH(AT_TILE_AT(0), 0)
         AT_LANDED();
         __syncthreads();
-        for (int t = t_lo; t <= t_hi; ++t) {
-            if (t < t_hi) AT_FETCH(t + 1, cur ^ 1)
+        for (int i = 0; i < n_tiles; ++i) {
+            const int t = AT_TILE_AT(i);
+            if (i + 1 < n_tiles) AT_FETCH(AT_TILE_AT(i + 1), cur ^ 1)
             AT_TILE(t)
             AT_LANDED();
             __syncthreads();
             cur ^= 1;
         }
     } else {
-        // chain c takes tiles t_lo + c, t_lo + c + CH, ...; every wave passes the same barriers, a chain
-        // whose tile lies past the last one loads that one again and computes nothing
-        const int iters = (t_hi - t_lo + CH) / CH;
-        int t = t_lo + chain;
-        AT_FETCH((t <= t_hi ? t : t_hi), 0)
+        // chain c takes walk steps c, c + CH, ...; every wave passes the same barriers, a chain
+        // whose step lies past the last one loads the last tile again and computes nothing
+        const int iters = (n_tiles - 1 + CH) / CH;
+        int i = chain;
+        AT_FETCH(AT_TILE_AT(i < n_tiles ? i : n_tiles - 1), 0)
         AT_LANDED();
         __syncthreads();
-        for (int it = 0; it < iters; ++it, t += CH) {
-            if (it + 1 < iters) AT_FETCH((t + CH <= t_hi ? t + CH : t_hi), cur ^ 1)
-            if (t <= t_hi) AT_TILE(t)
+        for (int it = 0; it < iters; ++it, i += CH) {
+            if (it + 1 < iters) AT_FETCH(AT_TILE_AT(i + CH < n_tiles ? i + CH : n_tiles - 1), cur ^ 1)
+            if (i < n_tiles) {
+                const int t = AT_TILE_AT(i);
+                AT_TILE(t)
+            }
             AT_LANDED();
             __syncthreads();
             cur ^= 1;
         }
     }
 #undef AT_TILE
+#undef AT_TILE_AT
 
     if (CH > 1) {
         // The second chain hands its running maximum, sum and accumulator over through LDS (the tiles
@@ -841,7 +858,7 @@ static size_t at_lds_bytes(int DC, int pages, int S, int chains = 1) {
 template <int AM_MERGE_THREADS>
 __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml, const int32_t* __restrict__ pos,
-    bf16_t* __restrict__ out, int out_stride, int nq, int D, int nsplit, int split_blocks, int window,
+    bf16_t* __restrict__ out, int out_stride, int nq, int D, int nsplit, int split_blocks, TlMask mask,
     const int32_t* __restrict__ seq_list, const int32_t* __restrict__ q_start, int sink) {
     __shared__ float wgt[AM_MAX_SPLITS];
     __shared__ float red_m[AM_MERGE_THREADS / 64], red_l[AM_MERGE_THREADS / 64];
@@ -849,10 +866,19 @@ __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     const int wrow = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int t = seq_list ? q_start[seq_list[wrow]] : wrow;   // listed one-token sequences: their row of the step
     const int p = pos[t];
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int lo = tl_mask_lo(mask, p);
     const int s_lo = (lo >> 5) / split_blocks, s_hi = (p >> 5) / split_blocks;
-    const int ns = s_hi - s_lo + 1;
-    const size_t base = ((size_t)wrow * nq + h) * nsplit + s_lo;
+    // the splits that hold kept first keys, [0, s_head), are visited ahead of those from s_lo on where the
+    // two do not touch: place s of the walk is split s below s_head and split s + s_shift from there on
+    int s_head = 0;
+    if (mask.first > 0 && lo > 0) {
+        s_head = ((mask.first - 1) >> 5) / split_blocks + 1;
+        if (s_head > s_lo) s_head = s_lo;
+    }
+    const int s_shift = s_lo - s_head;
+    const int ns = s_head + s_hi - s_lo + 1;
+#define AM_SPLIT_AT(S) ((S) < s_head ? (S) : (S) + s_shift)
+    const size_t base = ((size_t)wrow * nq + h) * nsplit;
     const int D4 = D >> 2, SG = AM_MERGE_THREADS / D4;      // D is 32, 64, 128 or 256
     const int d4 = tid % D4, sg = tid / D4;
     const float4* acc4 = reinterpret_cast<const float4*>(ws_o) + base * D4 + d4;
@@ -863,7 +889,7 @@ __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     for (int k = 0; k < AM_MERGE_AHEAD; ++k) {
         const int s = sg + k * SG;
         a[k] = zero4;
-        if (s < ns) a[k] = acc4[(size_t)s * D4];
+        if (s < ns) a[k] = acc4[(size_t)AM_SPLIT_AT(s) * D4];
     }
     float2 ml[AM_MAX_SPLITS / AM_MERGE_THREADS];
     float mx = -INFINITY;
@@ -871,7 +897,7 @@ __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     for (int j = 0; j < AM_MAX_SPLITS / AM_MERGE_THREADS; ++j) {
         const int s = tid + j * AM_MERGE_THREADS;
         ml[j] = make_float2(-INFINITY, 0.f);
-        if (s < ns) ml[j] = ml2[s];
+        if (s < ns) ml[j] = ml2[AM_SPLIT_AT(s)];
         mx = fmaxf(mx, ml[j].x);
     }
 #pragma unroll
@@ -907,7 +933,7 @@ __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
         }
     }
     for (int s = sg + AM_MERGE_AHEAD * SG; s < ns; s += SG) {
-        const float4 v = acc4[(size_t)s * D4];
+        const float4 v = acc4[(size_t)AM_SPLIT_AT(s) * D4];
         const float w = wgt[s];
         o4.x += v.x * w, o4.y += v.y * w, o4.z += v.z * w, o4.w += v.w * w;
     }
@@ -928,22 +954,24 @@ __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     }
 }
 
+#undef AM_SPLIT_AT
+
 template <int DC>
 static void launch_attn(int NT, dim3 grid, int wg_waves, hipStream_t stream, const bf16_t* q, int q_stride, const bf16_t* kc,
                         const bf16_t* vc, const int32_t* tables, int NB, const int32_t* q_start,
                         const int32_t* ctx_start, bf16_t* out, int out_stride, float* ws_o, float* ws_ml, int nq, int nkv,
-                        int bs, int window, float scale, int nsplit, int split_blocks, const int32_t* seq_list,
+                        int bs, TlMask mask, float scale, int nsplit, int split_blocks, const int32_t* seq_list,
                         int skip_single, int sink) {
     int bs_shift = -1;                               // pages of a power of two of tokens: a shift finds the page
     if ((bs & (bs - 1)) == 0)
         for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
     if (NT == 1)
         hipLaunchKernelGGL((attn_mfma_kernel<DC, 1>), grid, dim3(64 * wg_waves), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
-                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
+                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, mask, scale, nsplit,
                            split_blocks, seq_list, skip_single, sink);
     else
         hipLaunchKernelGGL((attn_mfma_kernel<DC, 2>), grid, dim3(64 * wg_waves), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
-                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
+                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, mask, scale, nsplit,
                            split_blocks, seq_list, skip_single, sink);
 }
 
@@ -962,17 +990,21 @@ static void launch_attn(int NT, dim3 grid, int wg_waves, hipStream_t stream, con
 // with skip_single != 0, which leaves sequences of one token out.
 // total_groups128: the sum over the sequences of ceil(n_s * G / 128), that kernel's grid.
 // sink != 0: one is added to the softmax's denominator (a key of score 0 that has no value).
+// window, chunk, keep_first: which keys a token sees (TlMask).
 extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
                                  const int32_t* pos, void* out, int out_stride, float* ws_o, float* ws_ml, int T, int S,
                                  int nq, int nkv, int d, int bs, int window, float scale, int NT, int max_tile_groups,
                                  int nsplit, int split_blocks, int shared, int total_groups128,
-                                 const int32_t* seq_list, int n_list, int skip_single, int sink, hipStream_t stream) {
+                                 const int32_t* seq_list, int n_list, int skip_single, int sink, int keep_first, int chunk,
+                                 hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_mfma: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_mfma: %d query heads are not a multiple of %d key/value heads", nq, nkv);
     TL_CHECK_ARG(d == 32 || d == 64 || d == 128 || d == 256, "tl_attention_mfma: head size %d is not one of 32, 64, 128, 256", d);
     TL_CHECK_ARG(bs >= 8 && bs % 8 == 0, "tl_attention_mfma: page size %d must be a multiple of 8", bs);
     TL_CHECK_ARG(NT == 1 || NT == 2, "tl_attention_mfma: NT=%d must be 1 or 2", NT);
+    TL_CHECK_ARG(window >= 0 && keep_first >= 0 && chunk >= 0, "tl_attention_mfma: negative window, chunk or kept first keys");
+    const TlMask mask{window, chunk, keep_first};
     TL_CHECK_ARG(nsplit >= 1 && nsplit <= AM_MAX_SPLITS && max_tile_groups >= 1,
                  "tl_attention_mfma: bad split count %d (at most %d) or group count", nsplit, AM_MAX_SPLITS);
     TL_CHECK_ARG(nsplit == 1 || (ws_o && ws_ml && pos && split_blocks >= 1),
@@ -1014,11 +1046,11 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
         if (chains == 2)                                                                                              \
             hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT, 2>), sgrid, dim3(2 * 64 * 8 / AT_NT), lds,    \
                                stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, \
-                               S, nq, nkv, bs, bs_shift, window, scale, skip_single, sink);                                 \
+                               S, nq, nkv, bs, bs_shift, mask, scale, skip_single, sink);                                 \
         else                                                                                                          \
             hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT, 1>), sgrid, dim3(64 * 8 / AT_NT), lds,        \
                                stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, \
-                               S, nq, nkv, bs, bs_shift, window, scale, skip_single, sink);                                 \
+                               S, nq, nkv, bs, bs_shift, mask, scale, skip_single, sink);                                 \
     } while (0)
         if (d == 32) TL_TILE_CASE(1);
         else if (d == 64) TL_TILE_CASE(2);
@@ -1029,25 +1061,25 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     }
     if (d == 32)
         launch_attn<1>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single, sink);
+                       ws_o, ws_ml, nq, nkv, bs, mask, scale, nsplit, split_blocks, seq_list, skip_single, sink);
     else if (d == 64)
         launch_attn<2>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single, sink);
+                       ws_o, ws_ml, nq, nkv, bs, mask, scale, nsplit, split_blocks, seq_list, skip_single, sink);
     else if (d == 128)
         launch_attn<4>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single, sink);
+                       ws_o, ws_ml, nq, nkv, bs, mask, scale, nsplit, split_blocks, seq_list, skip_single, sink);
     else
         launch_attn<8>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single, sink);
+                       ws_o, ws_ml, nq, nkv, bs, mask, scale, nsplit, split_blocks, seq_list, skip_single, sink);
     TL_CHECK_LAUNCH("tl_attention_mfma");
     if (nsplit > 1) {
         const int merge_rows = seq_list ? n_list : T;
         if (nsplit > 32)
             hipLaunchKernelGGL(attn_merge_kernel<256>, dim3(merge_rows, nq), dim3(256), 0, stream, ws_o, ws_ml, pos,
-                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window, seq_list, q_start, sink);
+                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, mask, seq_list, q_start, sink);
         else
             hipLaunchKernelGGL(attn_merge_kernel<128>, dim3(merge_rows, nq), dim3(128), 0, stream, ws_o, ws_ml, pos,
-                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window, seq_list, q_start, sink);
+                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, mask, seq_list, q_start, sink);
         TL_CHECK_LAUNCH("tl_attention_mfma merge");
     }
     return 0;

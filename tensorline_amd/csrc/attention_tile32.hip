@@ -220,7 +220,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int S, int nq, int nkv, int bs,
-    int bs_shift, int window, float scale, int skip_single, int sink) {
+    int bs_shift, TlMask mask, float scale, int skip_single, int sink) {
     constexpr int THREADS = WAVES * 64;
     constexpr int WGC = WAVES * 32;           // columns of a work-group
     constexpr int D = DC * 32, KS = D / 16, DT = D / 32;
@@ -275,24 +275,15 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
     // key range of the work-group and of this wave
     const int wg_last = ((wg_col0 + WGC < ncols) ? wg_col0 + WGC : ncols) - 1;
     const int khi = start + wg_last / G;
-    int klo = 0;
-    if (window > 0) {
-        klo = start + wg_col0 / G - window + 1;
-        if (klo < 0) klo = 0;
-    }
+    const int klo = tl_mask_lo(mask, start + wg_col0 / G);   // of the first column: no column's is lower
     const int t_lo = klo / T32_KEYS, t_hi = khi / T32_KEYS;
     int wk_lo = 1, wk_hi = 0, wk_full_hi = -1, wk_full_lo = 0;   // empty for a wave without columns
     if (wave_active) {
         const int w_last = ((col0 + 32 < ncols) ? col0 + 32 : ncols) - 1;
         wk_hi = start + w_last / G;           // the last key any column of the wave sees
         wk_full_hi = start + col0 / G;        // the last key every column of the wave sees
-        wk_lo = 0;
-        if (window > 0) {
-            wk_lo = start + col0 / G - window + 1;
-            if (wk_lo < 0) wk_lo = 0;
-            wk_full_lo = start + w_last / G - window + 1;     // the first key every column sees
-            if (wk_full_lo < 0) wk_full_lo = 0;
-        }
+        wk_lo = tl_mask_lo(mask, start + col0 / G);
+        wk_full_lo = tl_mask_lo(mask, start + w_last / G);    // the first key every column sees
     }
     // page ids into LDS
     {
@@ -335,7 +326,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
     const int gh = valid ? col - tok * G : 0;
     const int row_out = r0 + tok, head = kvh * G + gh;
     const int p_col = valid ? start + tok : T32_NO_COLUMN;
-    const int lo_col = (valid && window > 0 && p_col - window + 1 > 0) ? p_col - window + 1 : 0;
+    const int lo_col = valid ? tl_mask_lo(mask, p_col) : 0;
     uint4 qf[KS];
     {
         const bf16_t* qp = q + (size_t)row_out * q_stride + (size_t)head * D + h * 8;
@@ -456,7 +447,8 @@ extern "C" int tl_attention_tile32_columns(int waves) { return 32 * waves; }
 extern "C" int tl_attention_tile32(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                    const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
                                    void* out, int out_stride, int T, int S, int nq, int nkv, int d, int bs, int window,
-                                   float scale, int waves, int total_groups, int skip_single, int sink, hipStream_t stream) {
+                                   float scale, int waves, int total_groups, int skip_single, int sink, int chunk,
+                                   hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_tile32: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_tile32: %d query heads are not a multiple of %d key/value heads", nq, nkv);
     TL_CHECK_ARG(tl_attention_tile32_takes(d, bs, NB, S, waves),
@@ -469,7 +461,10 @@ extern "C" int tl_attention_tile32(const void* q, int q_stride, const void* k_ca
                  "tl_attention_tile32: %d key/value heads or %d column groups are more than a launch takes", nkv, total_groups);
     TL_CHECK_ARG(scale > 0.f, "tl_attention_tile32: the score scale %g must be positive", (double)scale);
     TL_CHECK_ARG((uint64_t)nkv * d * 2 * 8 < (1ull << 31), "tl_attention_tile32: a cache slot of %d heads is too wide", nkv);
+    TL_CHECK_ARG(window >= 0 && chunk >= 0, "tl_attention_tile32: negative window or chunk");
     if (T == 0 || S == 0 || total_groups == 0) return 0;
+    // windows and chunks; first keys kept in sight beyond them are left to the kernel of 16 columns per wave
+    const TlMask mask{window, chunk, 0};
     int bs_shift = 0;
     while ((1 << bs_shift) < bs) ++bs_shift;
     const size_t lds = t32_lds_bytes(d, NB, S);
@@ -477,7 +472,7 @@ extern "C" int tl_attention_tile32(const void* q, int q_stride, const void* k_ca
     const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
 #define T32_LAUNCH(DCV, WV)                                                                                             \
     hipLaunchKernelGGL((attn_tile32_kernel<DCV, WV>), grid, dim3(64 * WV), lds, stream, qq, q_stride, kk, vv, tables, NB, \
-                       q_start, ctx_start, (bf16_t*)out, out_stride, S, nq, nkv, bs, bs_shift, window, scale, skip_single, sink)
+                       q_start, ctx_start, (bf16_t*)out, out_stride, S, nq, nkv, bs, bs_shift, mask, scale, skip_single, sink)
     if (d == 64 && waves == 4) T32_LAUNCH(2, 4);
     else if (d == 64) T32_LAUNCH(2, 8);
     else if (waves == 4) T32_LAUNCH(4, 4);

@@ -103,6 +103,30 @@ struct TlNormArgs {
     int act;
 };
 
+// ---- which keys a token sees -------------------------------------------------------------------
+// Beside the causal rule (key <= p) a token at position p sees the keys from lo(p) on, and the first
+// `first` keys of its sequence wherever lo(p) lies:
+//   window > 0: lo = p - window + 1 (itself and the window - 1 keys before it);
+//   chunk > 0:  lo = the last multiple of chunk at or below p (positions count from the start of the
+//               sequence, not from where a step begins);
+//   both 0:     lo = 0.
+// lo never decreases with p.  Where lo(p) <= first the two ranges touch and lo is given as 0, so that a
+// gap between the kept first keys and lo exists exactly where lo > 0 and first > 0.
+struct TlMask {
+    int window, chunk, first;
+};
+__host__ __device__ __forceinline__ int tl_mask_lo(const TlMask& k, int p) {
+    int lo = 0;
+    if (k.window > 0 && p - k.window + 1 > lo) lo = p - k.window + 1;
+    if (k.chunk > 0) {
+        const int c = (p / k.chunk) * k.chunk;
+        lo = c > lo ? c : lo;
+    }
+    return lo <= k.first ? 0 : lo;
+}
+// a key below lo is hidden unless it is one of the kept first keys
+__device__ __forceinline__ bool tl_mask_hides(const TlMask& k, int key, int lo) { return key < lo && key >= k.first; }
+
 // ---- host side -----------------------------------------------------------------------------
 // Every C entry point returns 0 on success.  On failure it returns a non-zero code and leaves a
 // message that tl_last_error() hands out; nothing is launched in that case.

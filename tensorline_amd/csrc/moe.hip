@@ -88,6 +88,111 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
 }
 
+// Routing within the best groups.  Scores are s = sigmoid(logit).  The E experts form `groups` equal groups of
+// neighbours; a group's score is the sum of its two largest scores (of its one score, for groups of one);
+// only experts of the `keep` best groups can be chosen; of those the `top` with the largest scores are,
+// weighted by their scores divided by the sum of the chosen scores (+ 1e-20).  Among equals the lower index
+// wins, for groups and for experts.  A wave per token: lane l holds the scores of experts l, l + 64, ...
+// (at most 16 of them) and, as lane g, the score of group g (groups <= 64).
+__device__ __forceinline__ void moe_wave_best(float& bv, int& be) {   // the largest value over the wave, the lower index among equals
+    const int none = 0x7fffffff;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, 64);
+        const int oe = __shfl_xor(be, off, 64);
+        if (oe != none && (be == none || ov > bv || (ov == bv && oe < be))) {
+            bv = ov;
+            be = oe;
+        }
+    }
+}
+__global__ __launch_bounds__(256) void moe_route_grouped_kernel(const float* __restrict__ logits, int ldl,
+                                                                int32_t* __restrict__ ids, float* __restrict__ weights, int T,
+                                                                int E, int top, int groups, int keep) {
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const float* z = logits + (size_t)t * ldl;
+    const int none = 0x7fffffff, per = E / groups;
+    float s[MOE_MAX_EXPERTS / 64];
+#pragma unroll
+    for (int sl = 0; sl < MOE_MAX_EXPERTS / 64; ++sl) {
+        const int e = lane + 64 * sl;
+        s[sl] = e < E ? 1.0f / (1.0f + expf(-z[e])) : 0.f;
+    }
+    // group scores
+    float my_group = 0.f;
+    for (int g = 0; g < groups; ++g) {
+        float sum = 0.f;
+        int found = none;
+        for (int round = 0; round < 2; ++round) {
+            float bv = 0.f;
+            int be = none;
+#pragma unroll
+            for (int sl = 0; sl < MOE_MAX_EXPERTS / 64; ++sl) {
+                const int e = lane + 64 * sl;
+                if (e < E && e / per == g && e != found && (be == none || s[sl] > bv)) {
+                    bv = s[sl];
+                    be = e;
+                }
+            }
+            moe_wave_best(bv, be);
+            if (be == none) break;
+            sum += bv;
+            found = be;
+        }
+        if (lane == g) my_group = sum;
+    }
+    // the best groups
+    unsigned long long kept = 0ull;
+    for (int k = 0; k < keep; ++k) {
+        float bv = my_group;
+        int be = (lane < groups && !((kept >> lane) & 1ull)) ? lane : none;
+        moe_wave_best(bv, be);
+        kept |= 1ull << be;
+    }
+    // the best experts among them
+    unsigned taken = 0;
+    float my_val = 0.f;
+    int my_id = 0;
+    for (int c = 0; c < top; ++c) {
+        float bv = 0.f;
+        int be = none;
+#pragma unroll
+        for (int sl = 0; sl < MOE_MAX_EXPERTS / 64; ++sl) {
+            const int e = lane + 64 * sl;
+            if (e < E && !((taken >> sl) & 1u) && ((kept >> (e / per)) & 1ull) && (be == none || s[sl] > bv)) {
+                bv = s[sl];
+                be = e;
+            }
+        }
+        moe_wave_best(bv, be);
+        if ((be & 63) == lane) taken |= 1u << (be >> 6);
+        if (lane == c) {
+            my_val = bv;
+            my_id = be;
+        }
+    }
+    const float sum = tl_wave_sum(lane < top ? my_val : 0.f) + 1e-20f;
+    if (lane < top) {
+        ids[(size_t)t * top + lane] = my_id;
+        weights[(size_t)t * top + lane] = my_val / sum;
+    }
+}
+
+extern "C" int tl_moe_route_grouped(const float* logits, int ldl, int32_t* ids, float* weights, int T, int E, int top,
+                                    int groups, int keep, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && E > 0 && top > 0 && top <= MOE_MAX_TOP && E <= MOE_MAX_EXPERTS && ldl >= E,
+                 "tl_moe_route_grouped: bad sizes E=%d top=%d", E, top);
+    TL_CHECK_ARG(groups > 0 && groups <= 64 && E % groups == 0 && keep > 0 && keep <= groups && top <= keep * (E / groups),
+                 "tl_moe_route_grouped: %d experts in %d groups of which %d are kept do not give %d choices", E, groups, keep, top);
+    if (T == 0) return 0;
+    hipLaunchKernelGGL(moe_route_grouped_kernel, dim3(tl_ceil_div(T, 4)), dim3(256), 0, stream, logits, ldl, ids, weights, T, E,
+                       top, groups, keep);
+    TL_CHECK_LAUNCH("tl_moe_route_grouped");
+    return 0;
+}
+
 // mode 0: weights = softmax over the chosen logits; mode 1: weights = scale * sigmoid(chosen logit);
 // mode 2: weights = the chosen experts' shares of the softmax over all logits, not renormalised.
 extern "C" int tl_moe_route(const float* logits, int ldl, int32_t* ids, float* weights, int T, int E, int top, int mode,

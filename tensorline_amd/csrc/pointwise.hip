@@ -388,7 +388,7 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const T* __restrict__ q,
                                                         const int32_t* __restrict__ tables, int NB,
                                                         const int32_t* __restrict__ seq_of_token,
                                                         const int32_t* __restrict__ pos, T* __restrict__ out, int H, int D,
-                                                        int page, float scale) {
+                                                        int page, float scale, int window) {
     constexpr int E = WIDE_MAX_D / 64;
     __shared__ float sm[4], sl[4];
     __shared__ float sacc[4][WIDE_MAX_D];
@@ -405,7 +405,9 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const T* __restrict__ q,
         acc[e] = 0.f;
     }
     float m = -INFINITY, l = 0.f;
-    for (int j = w; j <= p; j += 4) {
+    // window > 0: keys from p - window + 1 on; a wave still takes the keys j with j % 4 == w
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    for (int j = (lo & ~3) + w + ((lo & 3) > w ? 4 : 0); j <= p; j += 4) {
         const T* krow = kc + ((size_t)table[j / page] * page + j % page) * D;
         float kv[E], dot = 0.f;
 #pragma unroll
@@ -441,23 +443,23 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(const T* __restrict__ q,
         float v = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) v += sacc[i][c] * f[i];
-        orow[c] = tl_from_float<T>(v / L);
+        orow[c] = tl_from_float<T>(L > 0.f ? v / L : 0.f);
     }
 }
 
 extern "C" int tl_attention_wide(const void* q, const void* k_cache, int dtype, const int32_t* tables, int NB,
                                  const int32_t* seq_of_token, const int32_t* pos, void* out, int T, int H, int D, int page,
-                                 float scale, hipStream_t stream) {
-    TL_CHECK_ARG(T >= 0 && H > 0 && H <= 65535 && D > 0 && D <= WIDE_MAX_D && page > 0 && NB > 0,
+                                 float scale, int window, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && H > 0 && H <= 65535 && D > 0 && D <= WIDE_MAX_D && page > 0 && NB > 0 && window >= 0,
                  "tl_attention_wide: bad sizes H=%d D=%d (rows of at most %d)", H, D, WIDE_MAX_D);
     if (T == 0) return 0;
     dim3 grid(T, H), block(256);
     if (dtype == TL_F32)
         hipLaunchKernelGGL(attn_wide_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_cache, tables, NB,
-                           seq_of_token, pos, (float*)out, H, D, page, scale);
+                           seq_of_token, pos, (float*)out, H, D, page, scale, window);
     else if (dtype == TL_BF16)
         hipLaunchKernelGGL(attn_wide_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache, tables, NB,
-                           seq_of_token, pos, (bf16_t*)out, H, D, page, scale);
+                           seq_of_token, pos, (bf16_t*)out, H, D, page, scale, window);
     else return tl_fail("tl_attention_wide: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("tl_attention_wide");
     return 0;
@@ -600,5 +602,141 @@ extern "C" int tl_diff_combine(const void* a, int lda, void* out, int dtype, int
                            lambda, eps, post);
     else return tl_fail("tl_diff_combine: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("tl_diff_combine");
+    return 0;
+}
+
+// ---- gated activations of a fused gate/up projection --------------------------------------------------------
+// gu [T, 2F] (gate columns first): out = act(gate) * up; kind 0: act = silu, kind 1: act = the tanh form of
+// gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).  float arithmetic.
+template <typename I, typename O>
+__global__ void glu_kernel(const I* __restrict__ gu, O* __restrict__ out, int T, int F, int kind) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)T * F) return;
+    const size_t t = i / F, c = i - t * F;
+    const float g = tl_to_float(gu[t * 2 * F + c]), u = tl_to_float(gu[t * 2 * F + F + c]);
+    out[i] = tl_from_float<O>((kind == 1 ? pw_gelu_tanh(g) : g * pw_sigmoid(g)) * u);
+}
+
+extern "C" int tl_glu(const void* gu, int in_dtype, void* out, int out_dtype, int T, int F, int kind, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && F > 0 && (kind == 0 || kind == 1), "tl_glu: bad sizes or unknown activation %d", kind);
+    if (T == 0) return 0;
+    dim3 grid((unsigned)(((size_t)T * F + 255) / 256)), block(256);
+#define GO(I, O) hipLaunchKernelGGL((glu_kernel<I, O>), grid, block, 0, stream, (const I*)gu, (O*)out, T, F, kind)
+    if (in_dtype == TL_F32 && out_dtype == TL_F32) GO(float, float);
+    else if (in_dtype == TL_F32 && out_dtype == TL_BF16) GO(float, bf16_t);
+    else if (in_dtype == TL_BF16 && out_dtype == TL_BF16) GO(bf16_t, bf16_t);
+    else return tl_fail("tl_glu: unsupported dtypes %d %d", in_dtype, out_dtype);
+#undef GO
+    TL_CHECK_LAUNCH("tl_glu");
+    return 0;
+}
+
+// ---- queries and keys normed per head, neighbouring pairs turned, the cache write ---------------------------
+// proj float [T, ldp] = [q: H*d | k: G*d | v: G*dv] (biases added already; no v columns with v_from_k).
+// Per token, for every query head and key head:
+//   * the head's d values are divided by their root mean square (eps inside the root) and multiplied by a
+//     weight per dimension that all heads share (wq [d], wk [d]; null: no norm);
+//   * then the pairs (2i, 2i + 1), i < rot / 2, are turned by the angle pos * freq[i], cosine and sine both
+//     times `mag` (freq null or rot 0: no rotation); the angle, its cosine and sine are float;
+//   * q goes to q_out [T, H*D], every head padded with zeros from d to D; k into the cache at `slot`
+//     ([pages, page, G, D], zeros from d to D); v with a page's tokens innermost ([pages, G, D, page], zeros
+//     from dv to D).  With v_from_k the values are the keys as projected: before norm and rotation.
+// A work-group per token; a wave takes a head at a time, a lane the pairs lane and lane + 64 of it (d <= 256).
+// A token's cosines and sines are computed once, into LDS, for all its heads.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_rotate_store_kernel(
+    const float* __restrict__ proj, int ldp, const int32_t* __restrict__ pos, const float* __restrict__ wq,
+    const float* __restrict__ wk, float eps, const float* __restrict__ freq, float mag, int rot,
+    const int32_t* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G,
+    int d, int dv, int D, int page, int v_from_k) {
+    __shared__ float cs[128], sn[128];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* row = proj + (size_t)t * ldp;
+    const float p = (float)pos[t];
+    for (int i = threadIdx.x; i < rot / 2; i += blockDim.x) {
+        const float a = p * freq[i];
+        cs[i] = cosf(a) * mag;
+        sn[i] = sinf(a) * mag;
+    }
+    __syncthreads();
+    const int slot = slots ? slots[t] : -1;
+    const size_t pg = slot >= 0 ? (size_t)slot / page : 0, within = slot >= 0 ? (size_t)slot % page : 0;
+    const int units = H + G + (v_from_k ? 0 : G);
+    for (int u = wave; u < units; u += 4) {
+        const bool is_q = u < H, is_k = !is_q && u < H + G;
+        const int head = is_q ? u : is_k ? u - H : u - H - G;
+        const int n = (is_q || is_k) ? d : dv;                   // the values the head has
+        const float* x = row + (is_q ? head * d : is_k ? H * d + head * d : (H + G) * d + head * dv);
+        float raw[4], y[4];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int c = 2 * (lane + 64 * j);
+            raw[2 * j] = c < n ? x[c] : 0.f;
+            raw[2 * j + 1] = c + 1 < n ? x[c + 1] : 0.f;
+        }
+        if (!is_q && slot < 0) continue;                         // nothing to write for this token (the same for the wave)
+        const float* w = is_q ? wq : is_k ? wk : nullptr;
+        float rstd = 1.0f;
+        if (w) {
+            const float ss = tl_wave_sum(raw[0] * raw[0] + raw[1] * raw[1] + raw[2] * raw[2] + raw[3] * raw[3]);
+            rstd = 1.0f / sqrtf(ss / (float)n + eps);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int i = lane + 64 * j, c = 2 * i;
+            float a = raw[2 * j], b = raw[2 * j + 1];
+            if (w) {
+                a = c < n ? a * rstd * w[c] : 0.f;
+                b = c + 1 < n ? b * rstd * w[c + 1] : 0.f;
+            }
+            if ((is_q || is_k) && c + 1 < rot) {
+                const float ra = a * cs[i] - b * sn[i], rb = b * cs[i] + a * sn[i];
+                a = ra;
+                b = rb;
+            }
+            y[2 * j] = a;
+            y[2 * j + 1] = b;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int c = 2 * (lane + 64 * j) + e;
+                if (c >= D) continue;
+                const T o = tl_from_float<T>(y[2 * j + e]);       // zeros beyond the head's values
+                if (is_q) {
+                    q_out[((size_t)t * H + head) * D + c] = o;
+                } else if (is_k) {
+                    k_cache[((size_t)slot * G + head) * D + c] = o;
+                    if (v_from_k) v_cache[((pg * G + head) * D + c) * page + within] = tl_from_float<T>(raw[2 * j + e]);
+                } else {
+                    v_cache[((pg * G + head) * D + c) * page + within] = o;
+                }
+            }
+        }
+    }
+}
+
+extern "C" int tl_head_norm_rotate_store(const float* proj, int ldp, const int32_t* pos, const float* wq, const float* wk,
+                                         float eps, const float* freq, float mag, int rot, const int32_t* slots, void* q_out,
+                                         void* k_cache, void* v_cache, int dtype, int T, int H, int G, int d, int dv, int D,
+                                         int page, int v_from_k, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && H > 0 && G >= 0 && d > 0 && dv > 0 && D >= d && D >= dv && D <= 256 && page > 0,
+                 "tl_head_norm_rotate_store: bad sizes H=%d G=%d d=%d dv=%d D=%d", H, G, d, dv, D);
+    TL_CHECK_ARG(rot >= 0 && rot % 2 == 0 && rot <= d && (rot == 0 || freq), "tl_head_norm_rotate_store: %d turned dimensions of %d", rot, d);
+    TL_CHECK_ARG(!v_from_k || dv == d, "tl_head_norm_rotate_store: values that are the keys have the keys' size");
+    TL_CHECK_ARG((wq == nullptr) == (wk == nullptr), "tl_head_norm_rotate_store: queries and keys are normed together or not at all");
+    TL_CHECK_ARG(ldp >= (H + G) * d + (v_from_k ? 0 : G * dv), "tl_head_norm_rotate_store: the projection's rows are too short");
+    TL_CHECK_ARG(G == 0 || (slots && k_cache && v_cache), "tl_head_norm_rotate_store: keys need their cache");
+    if (T == 0) return 0;
+    dim3 grid(T), block(256);
+#define GO(TT)                                                                                                         \
+    hipLaunchKernelGGL(head_norm_rotate_store_kernel<TT>, grid, block, 0, stream, proj, ldp, pos, wq, wk, eps, freq, mag, \
+                       rot, slots, (TT*)q_out, (TT*)k_cache, (TT*)v_cache, H, G, d, dv, D, page, v_from_k)
+    if (dtype == TL_F32) GO(float);
+    else if (dtype == TL_BF16) GO(bf16_t);
+    else return tl_fail("tl_head_norm_rotate_store: unknown dtype %d", dtype);
+#undef GO
+    TL_CHECK_LAUNCH("tl_head_norm_rotate_store");
     return 0;
 }

@@ -65,7 +65,7 @@ class ModelRunner:
         slots = [cache.state_slot(e.rid) for e in entries]
         packed = pack_batch(entries, tables, slots, cache.page_size, ngroups, cache.scratch_page,
                             self.model.vocab_size, pad_seqs=pad_seqs, pad_nb=pad_nb, scratch_slot=cache.scratch_slot,
-                            windowed=[g.window > 0 for g in cache.groups], vectors=self._vectors)
+                            windowed=[g.trims for g in cache.groups], vectors=self._vectors)
         packed.facts.fit_context = self.fit_context
         return packed
 

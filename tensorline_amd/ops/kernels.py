@@ -786,14 +786,17 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     q_start: torch.Tensor | None = None, ctx_start: torch.Tensor | None = None, plan=None,
                     path: str | None = None, split_keys: int | None = None,
                     single_seqs: torch.Tensor | None = None, route_singles: bool | None = None,
-                    sink: bool = False) -> torch.Tensor:
+                    sink: bool = False, keep_first: int = 0, chunk: int = 0) -> torch.Tensor:
     """Causal attention of each token over the cached keys of its sequence.
 
     ``q``: [T, >= nq*d] with the query heads in the first nq*d columns (row stride free);
     ``tables``: int32 [S, NB] page ids; ``seq_of_token``, ``pos``: int32 [T]; ``plan``: the step's
     host-side facts (``max_context``, ``max_query_len``, ``decode_only``, ``num_seqs``, ``q_lens``,
     ``starts``, ``fit_context``).  ``window`` > 0
-    limits a token at position p to keys [p - window + 1, p].  ``sink`` adds one to the softmax's
+    limits a token at position p to keys [p - window + 1, p]; ``chunk`` > 0 to the keys from the last
+    multiple of ``chunk`` at or below p on (positions count from the start of the sequence); with
+    ``keep_first`` > 0 the first ``keep_first`` keys of the sequence stay in sight wherever those ranges
+    begin.  ``sink`` adds one to the softmax's
     denominator (a key of score 0 that has no value): ``p_j = exp(s_j) / (1 + sum exp(s))``.  Returns [T, nq*d].
 
     bfloat16 with a head size of 32, 64 or 128 and pages of a multiple of 8 tokens runs on the
@@ -817,6 +820,10 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _check(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= num_heads * head_dim, "paged_attention: bad query layout")
     _check_caches(k_cache, v_cache, q.dtype, num_kv_heads, head_dim, "paged_attention")
     _check(tables.dim() == 2 and tables.dtype == torch.int32 and tables.is_contiguous(), "paged_attention: bad page table")
+    window, keep_first, chunk = int(window or 0), int(keep_first or 0), int(chunk or 0)
+    _check(window >= 0 and keep_first >= 0 and chunk >= 0, "paged_attention: a window, a chunk and kept first keys are not negative")
+    if not (window or chunk):
+        keep_first = 0                     # every key is in sight anyway
     _i32(seq_of_token, "seq_of_token", T)
     _i32(pos, "pos", T)
     if out is None:
@@ -850,7 +857,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                       _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws[:n_o]), _ptr(ws[n_o:]), T, S,
                       num_heads, num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt1,
                       -(-G // (16 * nt1)), nsplit, max(split_len // 32, 1), 0, 0, _ptr(single_seqs), len(singles), 0,
-                      int(bool(sink)), _stream())
+                      int(bool(sink)), keep_first, chunk, _stream())
                 skip_single = 1
         q_lens = [n for n in plan.q_lens if n > 1] if skip_single else plan.q_lens
         nt = 1 if plan.max_query_len * G <= 16 or head_dim == 256 else 2
@@ -874,7 +881,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
             ws_o, ws_ml = ws[:T * num_heads * nsplit * head_dim], ws[T * num_heads * nsplit * head_dim:]
         waves = 8 if path == "mfma-tile32" else _tile32_waves(plan.q_lens, plan.starts, num_heads) if path in (None, "mfma") else 0
-        if (waves and nt == 2 and nsplit == 1 and total128 > 0
+        if (waves and nt == 2 and nsplit == 1 and total128 > 0 and not keep_first      # kept first keys: the other kernel
                 and library().tl_attention_tile32_takes(head_dim, page, tables.shape[1], S, waves)):
             # prompt portions behind many keys, head size 64 or 128: 32 columns per wave on the 32x32
             # matrix-core instruction, work-groups of 256 columns
@@ -882,14 +889,14 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             total = sum(-(-n * G // cols) for n in q_lens) + pads
             _call("tl_attention_tile32", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
                   _ptr(q_start), _ptr(ctx_start), _ptr(out), o_stride, T, S, num_heads, num_kv_heads, head_dim, page,
-                  int(window), ctypes.c_float(scale), waves, total, skip_single, int(bool(sink)), _stream())
+                  int(window), ctypes.c_float(scale), waves, total, skip_single, int(bool(sink)), chunk, _stream())
             return out
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
               0 if path == "mfma-direct" else _tile16_chains(total128, num_kv_heads, path, plan.max_context), total128,
               _ptr(None), 0,
-              skip_single, int(bool(sink)), _stream())
+              skip_single, int(bool(sink)), keep_first, chunk, _stream())
         return out
     # The any-shape kernel tiles each sequence's tokens: it needs the first row of every sequence and the
     # most tokens one of them brings.  The engine has both; a bare call derives them from seq_of_token.
@@ -922,7 +929,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
           _ptr(q_start), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, S, max(max_query_len, 1), num_heads,
-          num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nsplit, split_len, _ptr(ws), int(bool(sink)), _stream())
+          num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nsplit, split_len, _ptr(ws), int(bool(sink)),
+          keep_first, chunk, _stream())
     return out
 
 
@@ -1064,6 +1072,22 @@ def clamp_glu(gate_up: torch.Tensor, limit: float, alpha: float, out_dtype: torc
     return out
 
 
+GLU_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def glu(gate_up: torch.Tensor, activation: str, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """For a fused [T, 2F] projection (gate columns first): ``act(gate) * up`` [T, F], ``act`` "silu" or
+    "gelu_tanh" (``0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``), computed in float32."""
+    _check(activation in GLU_ACTIVATIONS, f"glu: unknown activation {activation!r}")
+    _on_gpu(gate_up)
+    _check(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "glu: input must be contiguous [T, 2F]")
+    T, F2 = gate_up.shape
+    out = torch.empty(T, F2 // 2, dtype=out_dtype or gate_up.dtype, device=gate_up.device)
+    _call("tl_glu", _ptr(gate_up), _code(gate_up, "glu in"), _ptr(out), _code(out, "glu out"), T, F2 // 2,
+          GLU_ACTIVATIONS[activation], _stream())
+    return out
+
+
 def gated_group_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, group: int, eps: float, gate_act: str,
                      out_dtype: torch.dtype) -> torch.Tensor:
     """``o`` float32 [T, N] in groups of ``group`` columns, each divided by its root mean square (eps
@@ -1158,11 +1182,11 @@ WIDE_ROW_MAX = 1024      # the widest cached row the plain wide-row attention ta
 
 
 def wide_row_attention(q: torch.Tensor, k_cache: torch.Tensor, tables: torch.Tensor, seq_of_token: torch.Tensor,
-                       pos: torch.Tensor, heads: int, scale: float) -> torch.Tensor:
+                       pos: torch.Tensor, heads: int, scale: float, window: int = 0) -> torch.Tensor:
     """Causal attention of ``heads`` query heads over one shared key/value head whose cached rows (key and
     value at once) are wider than the matrix-core kernels take: ``q`` [T, heads * D], ``k_cache`` [pages,
     page, 1, D] with D up to ``WIDE_ROW_MAX``.  Plain float arithmetic, a work-group per (token, head): for
-    sizes nothing else serves.  Returns [T, heads * D]."""
+    sizes nothing else serves.  ``window`` > 0: a token sees the last ``window`` keys only.  Returns [T, heads * D]."""
     _on_gpu(q, k_cache, tables, seq_of_token, pos)
     T = q.shape[0]
     _check(k_cache.dim() == 4 and k_cache.is_contiguous() and k_cache.shape[2] == 1 and k_cache.dtype == q.dtype,
@@ -1174,7 +1198,7 @@ def wide_row_attention(q: torch.Tensor, k_cache: torch.Tensor, tables: torch.Ten
     _i32(pos, "pos", T)
     out = torch.empty_like(q)
     _call("tl_attention_wide", _ptr(q), _ptr(k_cache), _code(q, "wide_row_attention"), _ptr(tables), tables.shape[1],
-          _ptr(seq_of_token), _ptr(pos), _ptr(out), T, heads, D, page, ctypes.c_float(scale), _stream())
+          _ptr(seq_of_token), _ptr(pos), _ptr(out), T, heads, D, page, ctypes.c_float(scale), int(window or 0), _stream())
     return out
 
 
@@ -1284,21 +1308,35 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, ctx, st
 
 # ---------------------------------------------------------------------------------------------
 # Routed experts
-ROUTER_WEIGHTINGS = {"softmax_top": 0, "sigmoid": 1, "softmax_all": 2}
+ROUTER_WEIGHTINGS = {"softmax_top": 0, "sigmoid": 1, "softmax_all": 2, "sigmoid_grouped": 3}
 
 
-def moe_route(logits: torch.Tensor, top: int, weighting: str = "softmax_top", scale: float = 1.0) -> tuple[torch.Tensor, torch.Tensor]:
+def moe_route(logits: torch.Tensor, top: int, weighting: str = "softmax_top", scale: float = 1.0, experts: int | None = None,
+              groups: int = 1, keep: int = 1) -> tuple[torch.Tensor, torch.Tensor]:
     """Per row of float32 ``logits`` [T, E]: the ``top`` largest (lowest index first among equals), as
     int32 ids [T, top], and their weights, float32 [T, top]: the softmax over those alone
     (``weighting`` "softmax_top"), ``scale * sigmoid(logit)`` of each, not renormalised ("sigmoid"), or their
-    shares of the softmax over all E logits, not renormalised ("softmax_all")."""
+    shares of the softmax over all E logits, not renormalised ("softmax_all").  "sigmoid_grouped": scores are
+    ``sigmoid(logit)``; the experts form ``groups`` equal groups of neighbours, a group's score is the sum of its
+    two largest scores, only experts of the ``keep`` best groups can be chosen, and the chosen experts' weights are
+    their scores divided by their sum.  ``experts``: the first so many columns of ``logits`` are the router's
+    (default: all of them)."""
     _check(weighting in ROUTER_WEIGHTINGS, f"moe_route: unknown weighting {weighting!r}")
     _on_gpu(logits)
     T, E = logits.shape
+    if experts is not None:
+        _check(0 < experts <= E, "moe_route: more experts than columns")
+        E = int(experts)
     _check(logits.dtype == torch.float32 and logits.stride(1) == 1, "moe_route: logits must be float32 [T, E]")
     ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     weights = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    _call("tl_moe_route", _ptr(logits), logits.stride(0) if T > 1 else E, _ptr(ids), _ptr(weights), T, E, int(top),
+    ldl = logits.stride(0) if T > 1 else logits.shape[1]
+    if weighting == "sigmoid_grouped":
+        _check(groups > 0 and E % groups == 0 and 0 < keep <= groups and top <= keep * (E // groups) and groups <= 64,
+               f"moe_route: {E} experts in {groups} groups of which {keep} are kept do not give {top} choices")
+        _call("tl_moe_route_grouped", _ptr(logits), ldl, _ptr(ids), _ptr(weights), T, E, int(top), int(groups), int(keep), _stream())
+        return ids, weights
+    _call("tl_moe_route", _ptr(logits), ldl, _ptr(ids), _ptr(weights), T, E, int(top),
           ROUTER_WEIGHTINGS[weighting], ctypes.c_float(scale), _stream())
     return ids, weights
 
@@ -1435,6 +1473,45 @@ def qk_norm_store(proj: torch.Tensor, pos: torch.Tensor, q_weight: torch.Tensor 
     _call("tl_qk_norm_store", _ptr(proj), proj.stride(0) if T > 1 else proj.shape[1], _ptr(pos), _ptr(q_weight), _ptr(k_weight),
           ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every), _ptr(slots), _ptr(q), _ptr(k_cache), _ptr(v_cache),
           _code(q, "qk_norm_store"), T, heads, kv_heads, dim, vdim, D, page, _stream())
+    return q
+
+
+def head_norm_rotate_store(proj: torch.Tensor, pos: torch.Tensor, q_weight: torch.Tensor | None, k_weight: torch.Tensor | None,
+                           eps: float, freq: torch.Tensor | None, mag: float, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                           slots: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, values_from_keys: bool,
+                           out_dtype: torch.dtype) -> torch.Tensor:
+    """What lies between a fused q/k(/v) projection and attention, in one pass per token.  ``proj`` float32 [T,
+    heads*dim + kv_heads*dim (+ kv_heads*vdim)] (biases added).  Every query head and key head is RMS-normed over
+    its ``dim`` values with a weight per dimension that all heads share (float32 [dim]; both None: no norm), then
+    neighbouring pairs (2i, 2i + 1) of its first ``2 len(freq)`` dimensions are turned by ``pos * freq[i]``, cosine and
+    sine times ``mag`` (``freq`` None: no rotation).  Keys and values go into the cache pages at ``slots`` (``k_cache``
+    [pages, page, kv_heads, D], ``v_cache`` [pages, kv_heads, D, page]), heads padded with zeros to D.
+    ``values_from_keys``: there are no value columns; a key head's values are its keys as projected, before norm and
+    rotation.  Returns the queries [T, heads * D] in ``out_dtype``."""
+    _on_gpu(proj, pos, q_weight, k_weight, freq, k_cache, v_cache, slots)
+    T = proj.shape[0]
+    D, page = k_cache.shape[3], k_cache.shape[1]
+    cols = (heads + kv_heads) * dim + (0 if values_from_keys else kv_heads * vdim)
+    _check(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= cols,
+           "head_norm_rotate_store: bad projection")
+    _check_caches(k_cache, v_cache, out_dtype, kv_heads, D, "head_norm_rotate_store")
+    _check(dim <= D <= 256 and vdim <= D and (not values_from_keys or vdim == dim), "head_norm_rotate_store: head sizes do not fit the cache's")
+    _i32(pos, "pos", T)
+    _i32(slots, "slots", T)
+    _check((q_weight is None) == (k_weight is None), "head_norm_rotate_store: queries and keys are normed together or not at all")
+    if q_weight is not None:
+        _f32(q_weight, "head_norm_rotate_store q weight", dim)
+        _f32(k_weight, "head_norm_rotate_store k weight", dim)
+    rot = 0
+    if freq is not None:
+        rot = 2 * freq.numel()
+        _f32(freq, "head_norm_rotate_store frequencies", rot // 2)
+        _check(0 < rot <= dim, "head_norm_rotate_store: more turned dimensions than a head has")
+    q = torch.empty(T, heads * D, dtype=out_dtype, device=proj.device)
+    _call("tl_head_norm_rotate_store", _ptr(proj), proj.stride(0) if T > 1 else proj.shape[1], _ptr(pos), _ptr(q_weight),
+          _ptr(k_weight), ctypes.c_float(eps), _ptr(freq), ctypes.c_float(mag), rot, _ptr(slots), _ptr(q), _ptr(k_cache),
+          _ptr(v_cache), _code(q, "head_norm_rotate_store"), T, heads, kv_heads, dim, vdim, D, page,
+          1 if values_from_keys else 0, _stream())
     return q
 
 

@@ -9,6 +9,11 @@ Other designs change the weights (``weighting`` "sigmoid": each chosen expert by
 softmax over all experts, not renormalised), leave the router without bias, use the plain gated
 activation ``silu(g) * u`` (``activation`` "swiglu": no limit, alpha 1, nothing added to u), or have
 experts without gate, ``W_down relu(W_up h)^2`` (``activation`` "relu2": tensors e<i>.up / .down only).
+``weighting`` "sigmoid_grouped": scores are ``sigmoid(z)``; the experts form ``groups`` equal groups of neighbours, a
+group's score is the sum of its two largest scores, only experts of the ``keep_groups`` best groups can be chosen,
+and the chosen experts' weights are their scores divided by their sum.  A shared expert has the experts' activation
+(its ``limit`` only with the clamped one) and, with ``shared`` = {ff, gate: True}, is multiplied by
+``sigmoid(W_sg h)``, one number per token (``shared.sg`` [1, width]), before it is added.
 
 The experts' matrices are stacked ([experts, 2 ff, width] gate over up, [experts, width, ff]); a
 step's (token, choice) pairs are ordered by expert on the device and both products run as one
@@ -30,12 +35,13 @@ from tensorline_amd.parts.spec import TensorDecl
 class RoutedExperts(Part):
     """Parameters: ``experts``, ``top``, ``ff`` and ``limit`` of an expert, ``shared`` = {ff, limit} or
     None, ``alpha`` of the gate's sigmoid; ``weighting`` ("softmax_top", "sigmoid" or "softmax_all"),
-    ``router_scale``, ``router_bias``, ``activation`` ("clamped_glu", "swiglu" or "relu2").  Tensors under the prefix: router,
-    router.b, e<i>.gate / .up / .down, shared.gate / .up / .down."""
+    ``router_scale``, ``router_bias``, ``activation`` ("clamped_glu", "swiglu" or "relu2"), ``groups`` and ``keep_groups``
+    (with the weighting "sigmoid_grouped").  Tensors under the prefix: router,
+    router.b, e<i>.gate / .up / .down, shared.gate / .up / .down / .sg."""
 
     def __init__(self, hidden_size, prefix, dtype, device, experts: int, top: int, ff: int, limit: float | None = None,
                  shared: dict | None = None, alpha: float = 1.702, weighting: str = "softmax_top", router_scale: float = 1.0,
-                 router_bias: bool = True, activation: str = "clamped_glu"):
+                 router_bias: bool = True, activation: str = "clamped_glu", groups: int = 1, keep_groups: int | None = None):
         super().__init__(hidden_size, prefix, dtype, device)
         if activation not in ("clamped_glu", "swiglu", "relu2") or weighting not in kernels.ROUTER_WEIGHTINGS:
             raise ValueError(f"{prefix}: unknown activation {activation!r} or weighting {weighting!r}")
@@ -46,9 +52,18 @@ class RoutedExperts(Part):
             if limit is None:
                 raise ValueError(f"{prefix}: the clamped activation needs its limit")
             self.shift = 1.0
-        if shared and activation != "clamped_glu":
-            raise ValueError(f"{prefix}: a shared expert comes with the clamped activation only")
+        if shared and activation == "relu2":
+            raise ValueError(f"{prefix}: a shared expert comes with a gated activation only")
+        self.activation = activation
         self.weighting, self.router_scale = weighting, float(router_scale)
+        self.groups = int(groups)
+        self.keep_groups = self.groups if keep_groups is None else int(keep_groups)
+        if self.groups <= 0 or int(experts) % self.groups or not 0 < self.keep_groups <= self.groups or self.groups > 64:
+            raise ValueError(f"{prefix}: {experts} experts do not form {groups} equal groups (at most 64) of which {keep_groups} are kept")
+        if self.groups > 1 and weighting != "sigmoid_grouped":
+            raise ValueError(f"{prefix}: groups of experts come with the weighting 'sigmoid_grouped'")
+        if int(top) > self.keep_groups * (int(experts) // self.groups):
+            raise ValueError(f"{prefix}: {top} choices are more than the {self.keep_groups} kept groups hold")
         self.experts, self.top, self.ff, self.limit, self.alpha = int(experts), int(top), int(ff), float(limit), float(alpha)
         if not 0 < self.top <= self.experts or self.top > 32 or self.experts > 1024:
             raise ValueError(f"{prefix}: top {self.top} of {self.experts} experts is not served (top <= 32, experts <= 1024)")
@@ -56,16 +71,21 @@ class RoutedExperts(Part):
                              bias_name=prefix + "router.b")
         self.gate_up = self.down = None
         self.shared_ff = int(shared["ff"]) if shared else 0
-        self.shared_limit = float(shared["limit"]) if shared else 0.0
+        self.shared_limit = float(shared.get("limit", float("inf"))) if shared else 0.0
+        self.shared_gated = bool(shared and shared.get("gate"))      # the shared expert times sigmoid(W_sg h), per token
         self._sg = self._su = self.shared_gate_up = self.shared_down = None
         if shared:
             p = prefix + "shared."
             self._sg = Linear(p + "gate", hidden_size, self.shared_ff, False, weight_name=p + "gate")
             self._su = Linear(p + "up", hidden_size, self.shared_ff, False, weight_name=p + "up")
             self.shared_down = Linear(p + "down", self.shared_ff, hidden_size, False, weight_name=p + "down")
+        self._token_gate = Linear(prefix + "shared.sg", hidden_size, 1, False, weight_name=prefix + "shared.sg") \
+            if self.shared_gated else None
 
     def tensors(self):
         out = dict(self.router.tensors())
+        if self._token_gate is not None:
+            out.update(self._token_gate.tensors())
         for e in range(self.experts):
             p = f"{self.prefix}e{e}."
             if self.gated:
@@ -79,7 +99,13 @@ class RoutedExperts(Part):
 
     def load(self, get: TensorGetter) -> None:
         self.router.load(get)
-        self.router.prepare()
+        if self._token_gate is not None:
+            # the gate's one row rides on the router's product: logits [T, experts | gate]
+            self._token_gate.load(get)
+            self.router = fuse_linears(self.prefix + "router_sg", [self.router, self._token_gate])
+            self._token_gate.weight = None
+        else:
+            self.router.prepare()
         name = lambda e, s: f"{self.prefix}e{e}.{s}"
         if self.gated:
             self.gate_up = torch.stack([torch.cat([get(name(e, "gate")), get(name(e, "up"))]) for e in range(self.experts)]).contiguous()
@@ -106,10 +132,18 @@ class RoutedExperts(Part):
         return [(self.shared_gate_up.weight, self.dtype), (self.shared_down.weight, torch.float32)]
 
     def forward(self, h, ctx):
-        ids, weights = kernels.moe_route(self.router(h, out_dtype=torch.float32), self.top, self.weighting, self.router_scale)
+        logits = self.router(h, out_dtype=torch.float32)
+        ids, weights = kernels.moe_route(logits, self.top, self.weighting, self.router_scale, experts=self.experts,
+                                         groups=self.groups, keep=self.keep_groups)
         shared = None
         if self.shared_down is not None:
-            act = kernels.clamp_glu(self.shared_gate_up(h, out_dtype=torch.float32), self.shared_limit, self.alpha, self.dtype)
+            gate_up = self.shared_gate_up(h, out_dtype=torch.float32)
+            if self.activation == "swiglu":
+                act = kernels.glu(gate_up, "silu", self.dtype)
+            else:
+                act = kernels.clamp_glu(gate_up, self.shared_limit, self.alpha, self.dtype)
             shared = self.shared_down(act, out_dtype=torch.float32)
+            if self.shared_gated:
+                kernels.head_gate(shared, logits[:, self.experts:self.experts + 1], 1)
         return kernels.moe_experts(h, self.gate_up, self.down, ids, weights, self.limit, self.alpha, shared, self.shift,
                                    gated=self.gated)

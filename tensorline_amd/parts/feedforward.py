@@ -16,10 +16,15 @@ from tensorline_amd.parts.registry import register_feed_forward
 
 @register_feed_forward("swiglu")
 class SwiGLU(Part):
-    def __init__(self, hidden_size, prefix, dtype, device, intermediate_size: int, names: tuple | None = None):
+    def __init__(self, hidden_size, prefix, dtype, device, intermediate_size: int, names: tuple | None = None,
+                 activation: str = "silu"):
         """``names``: the checkpoint names of the gate, up and down matrices below the prefix where they are
-        not ``gate_proj.weight``, ``up_proj.weight`` and ``down_proj.weight``."""
+        not ``gate_proj.weight``, ``up_proj.weight`` and ``down_proj.weight``.  ``activation``: what the gate
+        passes, "silu" or "gelu_tanh" (the tanh form of GELU), computed in float32."""
         super().__init__(hidden_size, prefix, dtype, device)
+        if activation not in kernels.GLU_ACTIVATIONS:
+            raise ValueError(f"{prefix}: unknown activation {activation!r}; known: {', '.join(kernels.GLU_ACTIVATIONS)}")
+        self.activation = activation
         self.intermediate_size = int(intermediate_size)
         g, u, d = (prefix + n for n in names) if names else (None, None, None)
         self._gate = Linear(prefix + "gate_proj", hidden_size, self.intermediate_size, False, weight_name=g)
@@ -46,11 +51,15 @@ class SwiGLU(Part):
 
     @property
     def defers_norm(self) -> bool:
-        return self.gate_up.shuffled is not None and self.down.shuffled is not None
+        # the product that carries a norm has SiLU in its epilogue and no other activation
+        return self.activation == "silu" and self.gate_up.shuffled is not None and self.down.shuffled is not None
 
     keeps_share_sums = True
 
     def forward(self, h, ctx, sink=None, keep_shares: bool = False):
+        if self.activation != "silu":
+            act = kernels.glu(self.gate_up(h, out_dtype=torch.float32), self.activation, self.dtype)
+            return self.down(act, out_dtype=torch.float32, keep_shares=keep_shares)
         act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.streamed)
         return self.down(act, out_dtype=torch.float32, sink=sink, keep_shares=keep_shares)
 

@@ -16,17 +16,22 @@ from tensorline_amd.parts.spec import TensorDecl
 
 @register_norm("rmsnorm")
 class RMSNorm(Part):
-    def __init__(self, hidden_size, prefix, dtype, device, eps: float, name: str = "weight"):
+    def __init__(self, hidden_size, prefix, dtype, device, eps: float, name: str = "weight", around_zero: bool = False):
+        """``around_zero``: the checkpoint stores the weight's distance from one, ``x / rms(x) * (1 + w)``; the
+        one is added when the weight is loaded (in float32), and every kernel sees a plain weight."""
         super().__init__(hidden_size, prefix, dtype, device)
         self.eps = float(eps)
+        self.around_zero = bool(around_zero)
         self.name = prefix + name
         self.weight: torch.Tensor | None = None
 
     def tensors(self):
-        return {self.name: TensorDecl((self.hidden_size,), "one_plus_normal", 0.1, "float32")}
+        return {self.name: TensorDecl((self.hidden_size,), "normal" if self.around_zero else "one_plus_normal", 0.1, "float32")}
 
     def load(self, get: TensorGetter) -> None:
         self.weight = get(self.name)
+        if self.around_zero:
+            self.weight = (self.weight.to(torch.float32) + 1.0).contiguous()
 
     def weight_tensors(self):
         return [self.weight]

@@ -90,3 +90,4 @@ def _ensure_builtin() -> None:
     import tensorline_amd.parts.token_input  # noqa: F401
     import tensorline_amd.parts.parallel  # noqa: F401
     import tensorline_amd.parts.conv_attention  # noqa: F401
+    import tensorline_amd.parts.masked_attention  # noqa: F401

@@ -136,9 +136,13 @@ class CachePlane:
 @dataclass(frozen=True)
 class CacheNeed:
     """What a mixer keeps per token: one or more planes, for all earlier tokens (``window`` 0) or
-    for the last ``window`` of them.  Mixers with equal needs share a pool of pages."""
+    for the last ``window`` of them; with ``keep_first`` the first tokens of a sequence stay however far
+    the window has moved; with ``chunk`` only the tokens from the last multiple of ``chunk`` positions on
+    are needed.  Mixers with equal needs share a pool of pages."""
     planes: tuple[CachePlane, ...]
     window: int = 0
+    keep_first: int = 0
+    chunk: int = 0
 
     def __post_init__(self):
         names = [p.name for p in self.planes]
@@ -147,14 +151,30 @@ class CacheNeed:
 
     @property
     def kind(self) -> str:
-        return "window" if self.window > 0 else "full"
+        return "window" if self.window > 0 else "chunk" if self.chunk > 0 else "full"
+
+    @property
+    def trims(self) -> bool:
+        """Whether pages are given back while a request lives."""
+        return self.window > 0 or self.chunk > 0
+
+    def first_needed(self, computed: int) -> int:
+        """The first position (beyond the kept first tokens) that the token at position ``computed`` or any
+        later one still sees, once ``computed`` tokens are cached."""
+        first = 0
+        if self.window > 0:
+            first = max(first, computed - self.window + 1)
+        if self.chunk > 0:
+            first = max(first, (computed // self.chunk) * self.chunk)
+        return first
 
 
-def keys_and_values(num_kv_heads: int, head_dim: int, window: int = 0) -> CacheNeed:
+def keys_and_values(num_kv_heads: int, head_dim: int, window: int = 0, keep_first: int = 0, chunk: int = 0) -> CacheNeed:
     """The need of an attention mixer: keys ``k`` stored token by token, values ``v`` stored with
     the tokens of a page innermost (what the attention kernels read in one piece each)."""
     per_token = (int(num_kv_heads), int(head_dim))
-    return CacheNeed((CachePlane("k", per_token, "first"), CachePlane("v", per_token, "last")), int(window))
+    return CacheNeed((CachePlane("k", per_token, "first"), CachePlane("v", per_token, "last")), int(window),
+                     int(keep_first) if window else 0, int(chunk))
 
 
 @dataclass(frozen=True)

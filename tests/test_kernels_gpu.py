@@ -372,7 +372,8 @@ def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
 
 
 def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None,
-                    route_singles=None, pool_pages=None, spike_at=None, sink=False, spike_gain=4.0, score_shift=0.0):
+                    route_singles=None, pool_pages=None, spike_at=None, sink=False, spike_gain=4.0, score_shift=0.0,
+                    keep_first=0, chunk=0):
     """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries.
     pool_pages: the sequences' pages are the last ones of a pool of that many.  ``spike``: the key
     at position 1 (or at ``spike_at(position of the query)``, if that is a key at all) is made to
@@ -428,7 +429,8 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
                               torch.tensor(pos, dtype=torch.int32, device=DEV), nq, nkv, d, d ** -0.5, window=window,
                               q_start=torch.tensor(qs, dtype=torch.int32, device=DEV),
                               ctx_start=torch.tensor(plan.starts, dtype=torch.int32, device=DEV), plan=plan,
-                              path=path, split_keys=split_keys, single_seqs=single_seqs, route_singles=route_singles, sink=sink)
+                              path=path, split_keys=split_keys, single_seqs=single_seqs, route_singles=route_singles, sink=sink,
+                              keep_first=keep_first, chunk=chunk)
     if pool_pages:
         kc, vc, tables = kc[first:], vc[first:], tables - first
     kf, vf = kc.double().cpu().view(-1, nkv, d), vc.double().cpu().permute(0, 3, 1, 2).reshape(-1, nkv, d)
@@ -439,7 +441,10 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
         keys = torch.arange(n)
         rows = tcpu[s][keys // bs] * bs + keys % bs
         qs = q[t0:t0 + ql].double().cpu().view(ql, nq, d)
-        want[t0:t0 + ql] = plain.causal_attention(qs, kf[rows], vf[rows], d ** -0.5, window=window, q_offset=n - ql, sink=sink)
+        if keep_first or chunk:
+            want[t0:t0 + ql] = _masked_attention(qs, kf[rows], vf[rows], d ** -0.5, n - ql, window, keep_first, chunk)
+        else:
+            want[t0:t0 + ql] = plain.causal_attention(qs, kf[rows], vf[rows], d ** -0.5, window=window, q_offset=n - ql, sink=sink)
         t0 += ql
     return out.double().cpu().view(T, nq, d), want
 
@@ -632,6 +637,69 @@ def test_attention_one_token_sequences_beside_prompt_portions(heads, d, bs):
     short = _attention_case(dtype, heads[0], heads[1], d, bs, [500, 40, 9], [1, 40, 1], seed=12, route_singles=None)
     unrouted = _attention_case(dtype, heads[0], heads[1], d, bs, [500, 40, 9], [1, 40, 1], seed=12, route_singles=False)
     assert torch.equal(short[0], unrouted[0])                 # short contexts stay with the portions
+
+
+def _masked_attention(q, k, v, scale, q_offset, window, keep_first, chunk):
+    """q [n, nq, d] at positions q_offset.., k and v [keys, nkv, d]: the query at position i sees key j <= i if it
+    lies in the window (i - j < window) or among the first ``keep_first`` keys, and (with ``chunk``) in i's chunk."""
+    n, nq, d = q.shape
+    nkv = k.shape[1]
+    out = torch.zeros(n, nq, d, dtype=torch.float64)
+    for a in range(n):
+        i = q_offset + a
+        js = [j for j in range(i + 1) if (not window or i - j < window or j < keep_first) and (not chunk or j // chunk == i // chunk)]
+        for h in range(nq):
+            g = h // (nq // nkv)
+            w = torch.softmax(torch.stack([(q[a, h] * k[j, g]).sum() * scale for j in js]), 0)
+            out[a, h] = sum(w[x] * v[j, g] for x, j in enumerate(js))
+    return out
+
+
+MASK_PATHS = [("generic", torch.float32), ("generic", torch.bfloat16), ("mfma-direct", torch.bfloat16),
+              ("mfma-tile16", torch.bfloat16), ("mfma-tile16x2", torch.bfloat16), (None, torch.bfloat16)]
+
+
+@pytest.mark.parametrize("path,dtype", MASK_PATHS)
+@pytest.mark.parametrize("window,keep_first,chunk", [(40, 6, 0), (100, 70, 0), (33, 1, 0), (64, 64, 0), (0, 0, 48), (0, 0, 64), (0, 0, 7)])
+def test_attention_masks_in_prompt_portions(path, dtype, window, keep_first, chunk):
+    """A window beside which the first keys stay in sight, and chunks of positions, in every kernel that takes
+    prompt portions: portions that start at 0, behind cached tokens and in the middle of a window or chunk, beside
+    one-token sequences."""
+    lens, q_lens = [150, 9, 301, 77, 130], [150, 9, 40, 1, 1]
+    got, want = _attention_case(dtype, 4, 2, 64, 16, lens, q_lens, window=window, seed=31, path=path, keep_first=keep_first,
+                                chunk=chunk)
+    torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
+
+
+@pytest.mark.parametrize("path,dtype", [("generic", torch.float32), ("generic", torch.bfloat16), ("mfma-direct", torch.bfloat16),
+                                        (None, torch.bfloat16)])
+@pytest.mark.parametrize("split", [None, 64])
+@pytest.mark.parametrize("window,keep_first,chunk", [(40, 6, 0), (100, 70, 0), (200, 130, 0), (0, 0, 48), (0, 0, 128)])
+def test_attention_masks_in_one_token_steps(path, dtype, split, window, keep_first, chunk):
+    """The same masks where every sequence brings one token and the keys are split into runs: the kept first keys
+    in a run of their own, in the run the window starts in, and over several runs."""
+    lens = [700, 257, 256, 9, 357, 41, 130]
+    got, want = _attention_case(dtype, 6, 2, 32, 8, lens, None, window=window, seed=33, path=path, split_keys=split,
+                                keep_first=keep_first, chunk=chunk)
+    torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
+
+
+@pytest.mark.parametrize("path,dtype", MASK_PATHS)
+@pytest.mark.parametrize("where", ["first_in", "first_out", "window_in", "window_out", "chunk_in", "chunk_out"])
+def test_attention_masks_show_a_loud_key_on_the_right_side_of_every_edge(path, dtype, where):
+    """One key is made to match its query: the last kept first key and the one after it, the window's first key and
+    the one before it, a chunk's first key and the one before it.  Seen, it carries the sum, so an edge that is
+    off by one shows; prompt portions and one-token sequences."""
+    window, keep_first, chunk = (0, 0, 50) if where.startswith("chunk") else (37, 5, 0)
+    at = {"first_in": lambda p: keep_first - 1, "first_out": lambda p: keep_first, "window_in": lambda p: p - window + 1,
+          "window_out": lambda p: p - window, "chunk_in": lambda p: (p // chunk) * chunk,
+          "chunk_out": lambda p: (p // chunk) * chunk - 1}[where]
+    for lens, q_lens in (([160, 99, 300], [60, 1, 1]), ([120, 333, 64], None)):
+        if q_lens is None and path in ("mfma-tile16", "mfma-tile16x2"):
+            continue
+        got, want = _attention_case(dtype, 4, 2, 64, 16, lens, q_lens, window=window, seed=35, spike=True, path=path,
+                                    spike_at=at, keep_first=keep_first, chunk=chunk, spike_gain=6.0)
+        torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
