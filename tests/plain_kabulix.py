@@ -103,10 +103,11 @@ def mixer_attention(h, pos, W, p: str, m: dict, eps: float) -> torch.Tensor:
     v = k.clone()
     q = norm_plain(q, W[p + "q.norm"], eps)
     k = norm_plain(k, W[p + "k.norm"], eps)
-    freqs, mag = frequencies(m["rot"]["dims"], m["rot"]["base"], m["rot"].get("scaling"))
-    q, k = turn_pairs(q, pos, freqs, mag), turn_pairs(k, pos, freqs, mag)
-    size, first = m["mask"]["size"], m["mask"].get("keep_first", 0)
-    sees = lambda i, j: sees_window_and_first(i, j, size, first)
+    if m.get("rot"):
+        freqs, mag = frequencies(m["rot"]["dims"], m["rot"]["base"], m["rot"].get("scaling"))
+        q, k = turn_pairs(q, pos, freqs, mag), turn_pairs(k, pos, freqs, mag)
+    mask = m.get("mask")
+    sees = (lambda i, j: sees_window_and_first(i, j, mask["size"], mask.get("keep_first", 0))) if mask else (lambda i, j: j <= i)
     heads = [softmax_attention(q[:, a], k[:, a // (H // G)], v[:, a // (H // G)], pos, m["scale"], sees) for a in range(H)]
     return torch.cat(heads, 1) @ W[p + "o"].T
 
@@ -124,8 +125,8 @@ def mixer_latent(h, pos, W, p: str, m: dict, eps: float) -> torch.Tensor:
     q_turned = turn_pairs(q[:, :, d:], pos, freqs, mag)
     k_plain = (c @ W[p + "uk"].T).view(T, H, d)
     v = (c @ W[p + "uv"].T).view(T, H, dv)
-    size = m["mask"]["size"]
-    sees = lambda i, j: sees_window(i, j, size)
+    mask = m.get("mask")
+    sees = (lambda i, j: sees_window(i, j, mask["size"])) if mask else (lambda i, j: j <= i)
     heads = []
     for a in range(H):
         qa = torch.cat([q[:, a, :d], q_turned[:, a]], 1)
@@ -142,8 +143,8 @@ def mixer_chunked(h, pos, W, p: str, m: dict) -> torch.Tensor:
     q = (h @ W[p + "q"].T).view(T, H, d)
     k = (h @ W[p + "k"].T).view(T, G, d)
     v = (h @ W[p + "v"].T).view(T, G, dv)
-    size = m["mask"]["size"]
-    sees = lambda i, j: sees_chunk(i, j, size)
+    mask = m.get("mask")
+    sees = (lambda i, j: sees_chunk(i, j, mask["size"])) if mask else (lambda i, j: j <= i)
     gate = torch.sigmoid(h @ W[p + "g"].T)                   # [T, H]
     heads = [softmax_attention(q[:, a], k[:, a // (H // G)], v[:, a // (H // G)], pos, m["scale"], sees) * gate[:, a:a + 1]
              for a in range(H)]
@@ -171,18 +172,20 @@ def route(z: torch.Tensor, top: int, groups: int, keep: int) -> tuple[list[int],
     return chosen, [float(s[e]) / total for e in chosen]
 
 
-def ff_experts(h, W, p: str, mlp: dict, forced=None) -> torch.Tensor:
+def ff_experts(h, W, p: str, mlp: dict, forced=None, seen=None) -> torch.Tensor:
     """``forced``: per token the experts to use instead of the router's own choice (their weights still come from
-    the scores)."""
+    the scores).  ``seen``: a list that gets the router's logits [T, experts]."""
     r = mlp["router"]
     groups = (r.get("groups") or {}).get("count", 1)
     keep = (r.get("groups") or {}).get("keep", groups)
     out = torch.zeros_like(h)
     z = h @ W[p + "router"].T
+    if seen is not None:
+        seen.append(z.clone())
     for t in range(h.shape[0]):
         chosen, weights = route(z[t], r["top"], groups, keep)
         if forced is not None:
-            chosen = list(forced[t])
+            chosen = [int(e) for e in forced[t]]
             s = torch.sigmoid(z[t])
             total = sum(float(s[e]) for e in chosen) + 1e-20
             weights = [float(s[e]) / total for e in chosen]
@@ -193,33 +196,49 @@ def ff_experts(h, W, p: str, mlp: dict, forced=None) -> torch.Tensor:
     return out
 
 
-def router_margin(h, W, p: str, mlp: dict) -> torch.Tensor:
-    """Per token: how far apart the last chosen and the first rejected allowed score are (a small value is a close call)."""
+def is_close_call(z: torch.Tensor, taken, mlp: dict, slack: float) -> bool:
+    """Whether the experts ``taken`` are what the router chooses once every logit may move by up to ``slack``: tried
+    with theirs up and the others down, with one group at a time down and everything else up (a close call between
+    two groups neither of which holds a chosen expert), and with a few hundred random moves."""
     r = mlp["router"]
     groups = (r.get("groups") or {}).get("count", 1)
     keep = (r.get("groups") or {}).get("keep", groups)
-    z = h @ W[p + "router"].T
-    out = []
-    for t in range(h.shape[0]):
-        s = torch.sigmoid(z[t])
-        E, per = s.shape[0], s.shape[0] // groups
-        gs = sorted((sum(sorted((float(x) for x in s[g * per:(g + 1) * per]), reverse=True)[:2]) for g in range(groups)), reverse=True)
-        margin = gs[keep - 1] - gs[keep] if keep < groups else 1.0
-        chosen, _ = route(z[t], r["top"], groups, keep)
-        kept_groups = {e // per for e in chosen}
-        rest = [float(s[e]) for e in range(E) if e not in chosen and e // per in
-                set(sorted(range(groups), key=lambda g: (-sum(sorted((float(x) for x in s[g * per:(g + 1) * per]), reverse=True)[:2]), g))[:keep])]
-        if rest:
-            margin = min(margin, min(float(s[e]) for e in chosen) - max(rest))
-        out.append(margin)
-    return torch.tensor(out, dtype=F)
+    want = sorted(int(e) for e in taken)
+    E = z.shape[0]
+    per = E // groups
+    moves = [torch.full((E,), -slack, dtype=F)]
+    for e in want:
+        moves[0][e] = slack
+    for g in range(groups):
+        m = torch.full((E,), slack, dtype=F)
+        m[g * per:(g + 1) * per] = -slack
+        moves.append(m)
+        moves.append(torch.where(moves[0] > 0, moves[0], m))
+    gen = torch.Generator().manual_seed(0)
+    moves += [(torch.rand(E, generator=gen, dtype=F) * 2 - 1) * slack for _ in range(300)]
+    return any(sorted(route(z + m, r["top"], groups, keep)[0]) == want for m in moves)
+
+
+def mixer(kind: str, h, pos, W, p: str, m: dict, eps: float) -> torch.Tensor:
+    if kind == "attention":
+        return mixer_attention(h, pos, W, p, m, eps)
+    if kind == "latent_attention":
+        return mixer_latent(h, pos, W, p, m, eps)
+    if kind == "attention_2":
+        return mixer_chunked(h, pos, W, p, m)
+    raise ValueError(kind)
+
+
+def as_double(weights: dict) -> dict:
+    return {k: v.to(F) for k, v in weights.items() if v.dtype.is_floating_point}
 
 
 # ---- the model ------------------------------------------------------------------------------------
-def forward(config: dict, weights: dict, tokens, forced_experts=None, want_layers: bool = False):
+def forward(config: dict, weights: dict, tokens, forced_experts=None, want_layers: bool = False, router_logits=None):
     """Logits [T, vocab] of one sequence from position 0 (and the stream after every layer, if asked).
-    ``forced_experts``: {layer index: per token the experts to use}."""
-    W = {k: v.to(F) for k, v in weights.items() if v.dtype.is_floating_point}
+    ``forced_experts``: {layer index: per token the experts to use}; ``router_logits``: a dictionary that gets
+    {layer index: the router's logits [T, experts]}."""
+    W = as_double(weights)
     eps = config["norm"]["eps"]
     T = len(tokens)
     pos = list(range(T))
@@ -228,22 +247,17 @@ def forward(config: dict, weights: dict, tokens, forced_experts=None, want_layer
     for i, layer in enumerate(config["layers"]):
         p = f"l{i}."
         h = norm_around_zero(x, W[p + "norm1"], eps)
-        kind, m = layer["type"], layer["mixer"]
-        if kind == "attention":
-            x = x + mixer_attention(h, pos, W, p + "mix.", m, eps)
-        elif kind == "latent_attention":
-            x = x + mixer_latent(h, pos, W, p + "mix.", m, eps)
-        elif kind == "attention_2":
-            x = x + mixer_chunked(h, pos, W, p + "mix.", m)
-        else:
-            raise ValueError(kind)
+        x = x + mixer(layer["type"], h, pos, W, p + "mix.", layer["mixer"], eps)
         mlp = layer.get("mlp")
         if mlp is not None:
             h = norm_around_zero(x, W[p + "norm2"], eps)
             if mlp["kind"] == "dense":
                 x = x + gated_ff(h, W, p + "mlp.", gelu_tanh)
             else:
-                x = x + ff_experts(h, W, p + "mlp.", mlp, None if forced_experts is None else forced_experts.get(i))
+                seen = [] if router_logits is not None else None
+                x = x + ff_experts(h, W, p + "mlp.", mlp, None if forced_experts is None else forced_experts.get(i), seen)
+                if seen:
+                    router_logits[i] = seen[0]
         after.append(x.clone())
     logits = norm_around_zero(x, W["final.norm"], eps) @ W["embed"].T
     return (logits, torch.stack(after)) if want_layers else logits

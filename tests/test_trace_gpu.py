@@ -108,8 +108,8 @@ def test_mixed_steps_with_one_token_sequences_on_a_launch_of_their_own(setup, mo
     call = kernels._call
 
     def counting(fn, *args):
-        if fn == "tl_attention_mfma" and args[-5].value:       # the list of one-token sequences
-            routed.append(args[-4])
+        if fn == "tl_attention_mfma" and args[-7].value:       # the list of one-token sequences
+            routed.append(args[-6])
         return call(fn, *args)
     monkeypatch.setattr(kernels, "_call", counting)
     steps = helpers.steps_mixed(reqs)
