@@ -524,6 +524,48 @@ def make_zeganex_twin(size: str):
         rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768))
 
 
+# ---- the Kabulix design beside the dense decoder at equal size ----------------------------------------
+# Layer sizes that resemble real models of its kinds: windowed layers with heads of 128 in groups of four whose values
+# are their keys, half of a head rotated, four first tokens kept in sight; a latent layer with a latent of 192 + 64
+# rotated dimensions (a cached row of 256) and a gate per output column; a chunked layer with heads of 128 and a gate
+# per head; windows and chunks of 4,096 tokens (beyond the contexts measured, so that attention does the dense model's
+# work); a GELU feed-forward of three widths, experts of which 6 of 64 in 4 of 8 groups are used beside a gated shared
+# one.  Four layers (windowed + dense, latent + experts, windowed + experts, chunked + experts).  ``dense`` has the
+# same width, layers, vocabulary and attention heads, and a SwiGLU with the mean of the feed-forward weights a token reads.
+KABULIX_SIZES = {
+    "w1024": dict(width=1024, heads=8, experts=32, top=6, ff=512, shared_ff=512),
+    "w2048": dict(width=2048, heads=16, experts=64, top=6, ff=1408, shared_ff=1408),
+    "w4096": dict(width=4096, heads=32, experts=64, top=6, ff=2048, shared_ff=2048),
+}
+
+
+def make_kabulix_config(size: str, reach: int = 4096):
+    from tensorline_amd.config import KabulixConfig
+    z = KABULIX_SIZES[size]
+    W, H = z["width"], z["heads"]
+    windowed = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                "mask": {"size": reach, "keep_first": 4}, "rot": {"dims": 64, "base": 10000.0}}
+    latent = {"heads": H, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5, "mask": {"size": reach},
+              "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    chunked = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": reach}}
+    moe = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"], "groups": {"count": 8, "keep": 4}},
+           "expert": {"ff": z["ff"]}, "shared": {"ff": z["shared_ff"]}}
+    dense = {"kind": "dense", "ff": 3 * W}
+    layers = [{"type": "attention", "mixer": windowed, "mlp": dense}, {"type": "latent_attention", "mixer": latent, "mlp": moe},
+              {"type": "attention", "mixer": windowed, "mlp": moe}, {"type": "attention_2", "mixer": chunked, "mlp": moe}]
+    return KabulixConfig.from_dict({"architecture": "Kabulix", "vocab": HYBRID_VOCAB, "width": W, "norm": {"eps": 1e-6}, "layers": layers})
+
+
+def make_kabulix_twin(size: str):
+    from tensorline_amd.config import Qwen2Config
+    z = KABULIX_SIZES[size]
+    inter = (3 * z["width"] + 3 * (z["top"] * z["ff"] + z["shared_ff"])) // 4 // 128 * 128
+    return Qwen2Config.from_dict(dict(
+        architectures=["Qwen2ForCausalLM"], vocab_size=HYBRID_VOCAB, hidden_size=z["width"], intermediate_size=inter,
+        num_hidden_layers=4, num_attention_heads=z["heads"], num_key_value_heads=max(1, z["heads"] // 4), head_dim=128,
+        rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768))
+
+
 def profile_step(llm, entries_of, seed: int) -> dict:
     """Event time of every kernel of one eager step, summed per entry point (milliseconds), after a
     warm-up step of the same shape."""
@@ -554,7 +596,7 @@ def profile_step(llm, entries_of, seed: int) -> dict:
 
 def bench_hybrid(args, design: str = "samovik") -> int:
     """Prefill and decode throughput of a design at real layer sizes (``samovik``: HYBRID_SIZES, ``tumitar``:
-    TUMITAR_SIZES, ``zeganex``: ZEGANEX_SIZES) beside the dense decoder at equal size, and each step's time by kernel.  One JSON line;
+    TUMITAR_SIZES, ``zeganex``: ZEGANEX_SIZES, ``kabulix``: KABULIX_SIZES) beside the dense decoder at equal size, and each step's time by kernel.  One JSON line;
     the default benchmark is not run."""
     import torch
     table, make, make_twin, model_text = {
@@ -566,7 +608,11 @@ def bench_hybrid(args, design: str = "samovik") -> int:
                     "beside Qwen2 layers of equal width (4 layers)"),
         "zeganex": (ZEGANEX_SIZES, make_zeganex_config, make_zeganex_twin,
                     "Zeganex layer sizes (4 layers: rotary attention + dense, two-map attention + experts, rotary attention + "
-                    "experts, two-map attention on the second layer's cache + experts) beside Qwen2 layers of equal width (4 layers)")}[design]
+                    "experts, two-map attention on the second layer's cache + experts) beside Qwen2 layers of equal width (4 layers)"),
+        "kabulix": (KABULIX_SIZES, (lambda size: make_kabulix_config(size, args.reach)), make_kabulix_twin,
+                    "Kabulix layer sizes (4 layers: windowed attention with kept first tokens + dense, latent attention + experts, "
+                    "windowed attention + experts, chunked attention + experts; windows and chunks of %d tokens) beside Qwen2 "
+                    "layers of equal width (4 layers)" % args.reach)}[design]
 
     from tensorline_amd import LLM
     from tensorline_amd.engine.batch import StepEntry
@@ -658,6 +704,10 @@ def main() -> int:
     ap.add_argument("--zeganex", action="store_true",
                     help="the same for the Zeganex design (attention with short convolutions in two kinds, norms on both sides "
                          "of every branch, experts without gate)")
+    ap.add_argument("--kabulix", action="store_true",
+                    help="the same for the Kabulix design (windowed attention with kept first tokens, latent attention, chunked "
+                         "attention, experts chosen within groups beside a gated shared expert)")
+    ap.add_argument("--reach", type=int, default=4096, help="with --kabulix: tokens of its windows and chunks")
     ap.add_argument("--hybrid-sizes", default="", help="which of w1024,w2048,w4096 (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -671,6 +721,8 @@ def main() -> int:
         return bench_hybrid(args, "tumitar")
     if args.zeganex:
         return bench_hybrid(args, "zeganex")
+    if args.kabulix:
+        return bench_hybrid(args, "kabulix")
 
     import torch
 

@@ -99,7 +99,8 @@ struct TlNormArgs {
     float* ss_out;             // [tiles, ss_out_ld]: row `tile` gets the tile's sums of resid^2, one per row
     int ss_out_ld;
     // activation of a plain product's output, after the bias (the few-row kernel; no sink with it):
-    // 0 none, 1 the square of relu
+    // 0 none, 1 the square of relu; 2, in the gated two-tile form only: the tanh form of GELU passes the
+    // gate instead of SiLU
     int act;
 };
 

@@ -308,7 +308,10 @@ __global__ __launch_bounds__(MODE == MODE_SWIGLU ? 256 : 512) void gemm_skinny_k
             continue;
         }
         if (MODE == MODE_SWIGLU) {
-            v = v / (1.0f + expf(-v)) * u;
+            if (na.act == 2)                             // the tanh form of GELU passes the gate instead of SiLU
+                v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v))) * u;
+            else
+                v = v / (1.0f + expf(-v)) * u;
         } else if (bias) {
             v += bias[n];
         }
@@ -367,14 +370,14 @@ static int dispatch_skinny(const bf16_t* A, const uint4* Ws, const float* bias, 
 }
 
 // `norm` as the entry points take it: null for none.  A sink needs MODE_PLAIN (checked by the caller).
-static int check_norm(const TlNormArgs* norm, TlNormArgs* na, int M, int N, bool sink_allowed) {
+static int check_norm(const TlNormArgs* norm, TlNormArgs* na, int M, int N, bool sink_allowed, bool gated = false) {
     *na = TlNormArgs();
     if (!norm) return 0;
     *na = *norm;
     if (na->ss_in)
         TL_CHECK_ARG(na->ss_n > 0 && na->ss_ld >= M && na->dim > 0.f && na->eps >= 0.f,
                      "tl_gemm_skinny: bad owed-norm arguments (partials %d, stride %d)", na->ss_n, na->ss_ld);
-    TL_CHECK_ARG(na->act == 0 || (na->act == 1 && sink_allowed && !na->resid),
+    TL_CHECK_ARG(na->act == 0 || (na->act == 1 && sink_allowed && !na->resid) || (na->act == 2 && gated),
                  "tl_gemm_skinny: activation %d is not one a plain product without a sink applies", na->act);
     if (na->resid) {
         TL_CHECK_ARG(sink_allowed, "tl_gemm_skinny: only a plain product can add into the residual");
@@ -414,12 +417,13 @@ extern "C" int tl_gemm_skinny(const void* A, const void* Ws, const float* bias, 
 }
 
 // Ws: the shuffled copy of a [2I, K] matrix, rows [0, I) the gate and rows [I, 2I) the up projection;
-// I is a multiple of 16.  C [M, I] = silu(A Wg^T) * (A Wu^T), bfloat16.
+// I is a multiple of 16.  C [M, I] = silu(A Wg^T) * (A Wu^T), bfloat16 (norm->act == 2: the tanh form of GELU
+// in place of SiLU).
 extern "C" int tl_gemm_skinny_swiglu(const void* A, const void* Ws, void* C, int M, int I, int K, int lda, int ldc,
                                      const TlNormArgs* norm, hipStream_t stream) {
     if (int rc = check_skinny(A, Ws, C, M, 2 * I, K, lda, ldc)) return rc;
     TlNormArgs na;
-    if (int rc = check_norm(norm, &na, M, 2 * I, false)) return rc;
+    if (int rc = check_norm(norm, &na, M, 2 * I, false, true)) return rc;
     TL_CHECK_ARG(I % 16 == 0, "tl_gemm_skinny_swiglu: I=%d must be a multiple of 16", I);
     TL_CHECK_ARG(C && ldc >= I, "tl_gemm_skinny_swiglu: output row stride %d < I=%d", ldc, I);
     if (M == 0) return 0;

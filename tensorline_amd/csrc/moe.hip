@@ -106,6 +106,7 @@ __device__ __forceinline__ void moe_wave_best(float& bv, int& be) {   // the lar
         }
     }
 }
+template <int SL>      // scores a lane holds: 1 for up to 64 experts, 4 for up to 256, 16 beyond
 __global__ __launch_bounds__(256) void moe_route_grouped_kernel(const float* __restrict__ logits, int ldl,
                                                                 int32_t* __restrict__ ids, float* __restrict__ weights, int T,
                                                                 int E, int top, int groups, int keep) {
@@ -114,34 +115,36 @@ __global__ __launch_bounds__(256) void moe_route_grouped_kernel(const float* __r
     if (t >= T) return;
     const float* z = logits + (size_t)t * ldl;
     const int none = 0x7fffffff, per = E / groups;
-    float s[MOE_MAX_EXPERTS / 64];
+    const int nsl = (E + 63) >> 6;                         // slots in use: the same for the whole wave
+    float s[SL];
+    int grp[SL];
 #pragma unroll
-    for (int sl = 0; sl < MOE_MAX_EXPERTS / 64; ++sl) {
+    for (int sl = 0; sl < SL; ++sl) {
         const int e = lane + 64 * sl;
-        s[sl] = e < E ? 1.0f / (1.0f + expf(-z[e])) : 0.f;
+        const bool real = sl < nsl && e < E;
+        s[sl] = real ? 1.0f / (1.0f + expf(-z[e])) : -1.0f;
+        grp[sl] = real ? e / per : -1;
     }
-    // group scores
+    // group scores: per group the two largest scores over the wave (a butterfly over pairs (largest, second);
+    // scores lie in (0, 1), -1 stands for none), lane g keeps group g's
     float my_group = 0.f;
     for (int g = 0; g < groups; ++g) {
-        float sum = 0.f;
-        int found = none;
-        for (int round = 0; round < 2; ++round) {
-            float bv = 0.f;
-            int be = none;
+        float a1 = -1.0f, a2 = -1.0f;
 #pragma unroll
-            for (int sl = 0; sl < MOE_MAX_EXPERTS / 64; ++sl) {
-                const int e = lane + 64 * sl;
-                if (e < E && e / per == g && e != found && (be == none || s[sl] > bv)) {
-                    bv = s[sl];
-                    be = e;
-                }
+        for (int sl = 0; sl < SL; ++sl) {
+            if (sl < nsl && grp[sl] == g) {
+                const float v = s[sl];
+                a2 = fmaxf(a2, fminf(a1, v));
+                a1 = fmaxf(a1, v);
             }
-            moe_wave_best(bv, be);
-            if (be == none) break;
-            sum += bv;
-            found = be;
         }
-        if (lane == g) my_group = sum;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float b1 = __shfl_xor(a1, off, 64), b2 = __shfl_xor(a2, off, 64);
+            a2 = fmaxf(fminf(a1, b1), fmaxf(a2, b2));
+            a1 = fmaxf(a1, b1);
+        }
+        if (lane == g) my_group = fmaxf(a1, 0.f) + fmaxf(a2, 0.f);
     }
     // the best groups
     unsigned long long kept = 0ull;
@@ -159,11 +162,10 @@ __global__ __launch_bounds__(256) void moe_route_grouped_kernel(const float* __r
         float bv = 0.f;
         int be = none;
 #pragma unroll
-        for (int sl = 0; sl < MOE_MAX_EXPERTS / 64; ++sl) {
-            const int e = lane + 64 * sl;
-            if (e < E && !((taken >> sl) & 1u) && ((kept >> (e / per)) & 1ull) && (be == none || s[sl] > bv)) {
+        for (int sl = 0; sl < SL; ++sl) {
+            if (sl < nsl && grp[sl] >= 0 && !((taken >> sl) & 1u) && ((kept >> grp[sl]) & 1ull) && (be == none || s[sl] > bv)) {
                 bv = s[sl];
-                be = e;
+                be = lane + 64 * sl;
             }
         }
         moe_wave_best(bv, be);
@@ -187,8 +189,13 @@ extern "C" int tl_moe_route_grouped(const float* logits, int ldl, int32_t* ids, 
     TL_CHECK_ARG(groups > 0 && groups <= 64 && E % groups == 0 && keep > 0 && keep <= groups && top <= keep * (E / groups),
                  "tl_moe_route_grouped: %d experts in %d groups of which %d are kept do not give %d choices", E, groups, keep, top);
     if (T == 0) return 0;
-    hipLaunchKernelGGL(moe_route_grouped_kernel, dim3(tl_ceil_div(T, 4)), dim3(256), 0, stream, logits, ldl, ids, weights, T, E,
-                       top, groups, keep);
+#define GO(SLV)                                                                                                     \
+    hipLaunchKernelGGL(moe_route_grouped_kernel<SLV>, dim3(tl_ceil_div(T, 4)), dim3(256), 0, stream, logits, ldl, ids, \
+                       weights, T, E, top, groups, keep)
+    if (E <= 64) GO(1);
+    else if (E <= 256) GO(4);
+    else GO(MOE_MAX_EXPERTS / 64);
+#undef GO
     TL_CHECK_LAUNCH("tl_moe_route_grouped");
     return 0;
 }
@@ -610,22 +617,25 @@ extern "C" int tl_moe_gemm(const void* A, int a_dtype, int lda, const void* W, i
 
 // ---- the weighted sum per token ---------------------------------------------------------------------------------
 __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ weights,
-                                   const float* __restrict__ shared, float* __restrict__ out, int T, int N, int top) {
+                                   const float* __restrict__ shared, const float* __restrict__ shared_gate, int ldg,
+                                   float* __restrict__ out, int T, int N, int top) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)T * N) return;
     const size_t t = i / N, c = i - t * N;
     float sum = 0.f;
     for (int k = 0; k < top; ++k) sum += weights[t * top + k] * y[(t * top + k) * N + c];
-    if (shared) sum += shared[i];
+    if (shared) sum += shared_gate ? shared[i] * (1.0f / (1.0f + expf(-shared_gate[t * ldg]))) : shared[i];
     out[i] = sum;
 }
 
-extern "C" int tl_moe_combine(const float* y, const float* weights, const float* shared, float* out, int T, int N, int top,
-                              hipStream_t stream) {
-    TL_CHECK_ARG(T >= 0 && N > 0 && top > 0, "tl_moe_combine: bad sizes");
+// shared_gate (null: none): one logit per token with row stride ldg; the shared expert's row is multiplied by its
+// sigmoid before it is added.
+extern "C" int tl_moe_combine(const float* y, const float* weights, const float* shared, const float* shared_gate, int ldg,
+                              float* out, int T, int N, int top, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && N > 0 && top > 0 && (!shared_gate || (shared && ldg > 0)), "tl_moe_combine: bad sizes");
     if (T == 0) return 0;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)(((size_t)T * N + 255) / 256)), dim3(256), 0, stream, y, weights,
-                       shared, out, T, N, top);
+                       shared, shared_gate, ldg, out, T, N, top);
     TL_CHECK_LAUNCH("tl_moe_combine");
     return 0;
 }

@@ -641,8 +641,8 @@ extern "C" int tl_glu(const void* gu, int in_dtype, void* out, int out_dtype, in
 //   * q goes to q_out [T, H*D], every head padded with zeros from d to D; k into the cache at `slot`
 //     ([pages, page, G, D], zeros from d to D); v with a page's tokens innermost ([pages, G, D, page], zeros
 //     from dv to D).  With v_from_k the values are the keys as projected: before norm and rotation.
-// A work-group per token; a wave takes a head at a time, a lane the pairs lane and lane + 64 of it (d <= 256).
-// A token's cosines and sines are computed once, into LDS, for all its heads.
+// A work-group per token and four heads (of queries, keys or values, in that order); a wave takes one head, a lane
+// the pairs lane and lane + 64 of it (d <= 256).  A work-group computes the token's cosines and sines once, into LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_rotate_store_kernel(
     const float* __restrict__ proj, int ldp, const int32_t* __restrict__ pos, const float* __restrict__ wq,
@@ -662,7 +662,7 @@ __global__ __launch_bounds__(256) void head_norm_rotate_store_kernel(
     const int slot = slots ? slots[t] : -1;
     const size_t pg = slot >= 0 ? (size_t)slot / page : 0, within = slot >= 0 ? (size_t)slot % page : 0;
     const int units = H + G + (v_from_k ? 0 : G);
-    for (int u = wave; u < units; u += 4) {
+    for (int u = blockIdx.y * 4 + wave; u < units; u += units) {       // one head per wave; written as a loop for its early exits
         const bool is_q = u < H, is_k = !is_q && u < H + G;
         const int head = is_q ? u : is_k ? u - H : u - H - G;
         const int n = (is_q || is_k) ? d : dv;                   // the values the head has
@@ -729,7 +729,8 @@ extern "C" int tl_head_norm_rotate_store(const float* proj, int ldp, const int32
     TL_CHECK_ARG(ldp >= (H + G) * d + (v_from_k ? 0 : G * dv), "tl_head_norm_rotate_store: the projection's rows are too short");
     TL_CHECK_ARG(G == 0 || (slots && k_cache && v_cache), "tl_head_norm_rotate_store: keys need their cache");
     if (T == 0) return 0;
-    dim3 grid(T), block(256);
+    dim3 grid(T, tl_ceil_div(H + G + (v_from_k ? 0 : G), 4)), block(256);
+    TL_CHECK_ARG(grid.y <= 65535, "tl_head_norm_rotate_store: too many heads");
 #define GO(TT)                                                                                                         \
     hipLaunchKernelGGL(head_norm_rotate_store_kernel<TT>, grid, block, 0, stream, proj, ldp, pos, wq, wk, eps, freq, mag, \
                        rot, slots, (TT*)q_out, (TT*)k_cache, (TT*)v_cache, H, G, d, dv, D, page, v_from_k)

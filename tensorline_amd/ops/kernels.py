@@ -570,10 +570,27 @@ def tune_library_linear(rows: int, weight: torch.Tensor, out_dtype: torch.dtype,
 
 
 def swiglu_gate_up(h: torch.Tensor | NormedRows, gate_up_weight: torch.Tensor,
-                   shuffled: torch.Tensor | None = None) -> torch.Tensor:
+                   shuffled: torch.Tensor | None = None, activation: str = "silu") -> torch.Tensor:
     """``silu(h Wg^T) * (h Wu^T)`` for a fused [2I, K] weight (gate rows first): one kernel for
     few-row bfloat16 batches (it streams the ``shuffled`` copy), product then SiLU-multiply otherwise.
-    ``h`` may be :class:`NormedRows` (few-row kernel only)."""
+    ``h`` may be :class:`NormedRows` (few-row kernel only).  ``activation`` "gelu_tanh": the tanh form of GELU
+    passes the gate instead of SiLU (in the few-row kernel's epilogue, or by a pass over the float32 product)."""
+    _check(activation in GLU_ACTIVATIONS, f"swiglu_gate_up: unknown activation {activation!r}")
+    if activation != "silu":
+        _check(not isinstance(h, NormedRows), "swiglu_gate_up: only SiLU rides on a product that carries a norm")
+        M, K = h.shape
+        I = gate_up_weight.shape[0] // 2
+        lda = h.stride(0) if M > 1 else K
+        if h.dim() == 2 and h.stride(1) == 1 and _skinny_ok(h, shuffled, M, K, lda) and I % 16 == 0:
+            _on_gpu(h, gate_up_weight, shuffled)
+            _check(gate_up_weight.shape[1] == K and gate_up_weight.shape[0] % 2 == 0, "swiglu_gate_up: bad shapes")
+            _check_shuffled(shuffled, 2 * I, K)
+            out = torch.empty(M, I, dtype=h.dtype, device=h.device)
+            na = _NormArgs()
+            na.act = 2
+            _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(shuffled), _ptr(out), M, I, K, lda, I, ctypes.byref(na), _stream())
+            return out
+        return glu(linear(h, gate_up_weight, out_dtype=torch.float32, shuffled=shuffled), activation, h.dtype)
     owed = h if isinstance(h, NormedRows) else None
     if owed is not None:
         h = owed.rows
@@ -1348,14 +1365,15 @@ def moe_tile_rows(pairs: int, experts: int) -> int:
 
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
                 limit: float, alpha: float, shared: torch.Tensor | None = None, shift: float = 1.0,
-                gated: bool = True) -> torch.Tensor:
+                gated: bool = True, shared_gate: torch.Tensor | None = None) -> torch.Tensor:
     """``out[t] = sum_c weights[t, c] * expert_{ids[t, c]}(h[t]) (+ shared[t])`` in float32, where expert
     e is ``down[e] @ act(gate_up[e] @ h)`` with the gated activation ``g' sigmoid(alpha g') (u' + shift)``,
     ``g' = min(g, limit)``, ``u' = clamp(u, -limit, limit)`` (:func:`clamp_glu` has ``shift`` 1; an infinite
     ``limit`` with ``alpha`` 1 and ``shift`` 0 is ``silu(g) * u``).
     ``gate_up`` [E, 2F, K] (gate rows first), ``down`` [E, N, F]; ``h`` [T, K] in the weights' dtype.
-    ``gated`` False: experts without gate, ``down[e] @ relu(up[e] @ h)^2`` with ``gate_up`` = up [E, F, K]."""
-    _on_gpu(h, gate_up, down, ids, weights, shared)
+    ``gated`` False: experts without gate, ``down[e] @ relu(up[e] @ h)^2`` with ``gate_up`` = up [E, F, K].
+    ``shared_gate`` float32 [T, 1] (rows may be strided): ``shared[t]`` is multiplied by ``sigmoid(shared_gate[t])``."""
+    _on_gpu(h, gate_up, down, ids, weights, shared, shared_gate)
     T, K = h.shape
     E, F2, _ = gate_up.shape
     F, N, top = (F2 // 2 if gated else F2), down.shape[1], ids.shape[1]
@@ -1380,7 +1398,12 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids:
           _ptr(order), _ptr(tiles), max_tiles, BM, top, N, F, 0, ctypes.c_float(0.0), ctypes.c_float(0.0), ctypes.c_float(0.0),
           _stream())
     out = torch.empty(T, N, dtype=torch.float32, device=h.device)
-    _call("tl_moe_combine", _ptr(y), _ptr(weights), _ptr(shared), _ptr(out), T, N, top, _stream())
+    ldg = 0
+    if shared_gate is not None:
+        _check(shared is not None and shared_gate.dtype == torch.float32 and tuple(shared_gate.shape) == (T, 1),
+               "moe_experts: the shared expert's gate is float32 [T, 1]")
+        ldg = shared_gate.stride(0) if T > 1 else 1
+    _call("tl_moe_combine", _ptr(y), _ptr(weights), _ptr(shared), _ptr(shared_gate), ldg, _ptr(out), T, N, top, _stream())
     return out
 
 

@@ -137,13 +137,11 @@ class RoutedExperts(Part):
                                          groups=self.groups, keep=self.keep_groups)
         shared = None
         if self.shared_down is not None:
-            gate_up = self.shared_gate_up(h, out_dtype=torch.float32)
-            if self.activation == "swiglu":
-                act = kernels.glu(gate_up, "silu", self.dtype)
+            if self.activation == "swiglu":       # SiLU rides on the few-row product, as in the dense feed-forward
+                act = kernels.swiglu_gate_up(h, self.shared_gate_up.weight, self.shared_gate_up.streamed)
             else:
-                act = kernels.clamp_glu(gate_up, self.shared_limit, self.alpha, self.dtype)
+                act = kernels.clamp_glu(self.shared_gate_up(h, out_dtype=torch.float32), self.shared_limit, self.alpha, self.dtype)
             shared = self.shared_down(act, out_dtype=torch.float32)
-            if self.shared_gated:
-                kernels.head_gate(shared, logits[:, self.experts:self.experts + 1], 1)
+        token_gate = logits[:, self.experts:self.experts + 1] if self.shared_gated else None     # applied where it is added
         return kernels.moe_experts(h, self.gate_up, self.down, ids, weights, self.limit, self.alpha, shared, self.shift,
-                                   gated=self.gated)
+                                   gated=self.gated, shared_gate=token_gate)

@@ -58,7 +58,7 @@ class SwiGLU(Part):
 
     def forward(self, h, ctx, sink=None, keep_shares: bool = False):
         if self.activation != "silu":
-            act = kernels.glu(self.gate_up(h, out_dtype=torch.float32), self.activation, self.dtype)
+            act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.streamed, activation=self.activation)
             return self.down(act, out_dtype=torch.float32, keep_shares=keep_shares)
         act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.streamed)
         return self.down(act, out_dtype=torch.float32, sink=sink, keep_shares=keep_shares)
