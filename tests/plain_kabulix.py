@@ -83,10 +83,14 @@ def sees_chunk(i: int, j: int, size: int) -> bool:
     return j <= i and i // size == j // size
 
 
-def softmax_attention(q, k, v, pos, scale: float, sees) -> torch.Tensor:
+def sight(pos, sees) -> torch.Tensor:
+    """[T, T] of booleans: whether the token in row i sees the token in column j."""
+    T = len(pos)
+    return torch.tensor([[sees(int(pos[i]), int(pos[j])) for j in range(T)] for i in range(T)])
+
+
+def softmax_attention(q, k, v, mask, scale: float) -> torch.Tensor:
     """q [T, dk], k [T, dk], v [T, dv] of one head: row i is the softmax-weighted mean of the v_j it sees."""
-    T = q.shape[0]
-    mask = torch.tensor([[sees(int(pos[i]), int(pos[j])) for j in range(T)] for i in range(T)])
     s = (q @ k.T) * scale
     w = torch.softmax(s.masked_fill(~mask, float("-inf")), dim=1)
     return w @ v
@@ -108,7 +112,8 @@ def mixer_attention(h, pos, W, p: str, m: dict, eps: float) -> torch.Tensor:
         q, k = turn_pairs(q, pos, freqs, mag), turn_pairs(k, pos, freqs, mag)
     mask = m.get("mask")
     sees = (lambda i, j: sees_window_and_first(i, j, mask["size"], mask.get("keep_first", 0))) if mask else (lambda i, j: j <= i)
-    heads = [softmax_attention(q[:, a], k[:, a // (H // G)], v[:, a // (H // G)], pos, m["scale"], sees) for a in range(H)]
+    seen = sight(pos, sees)
+    heads = [softmax_attention(q[:, a], k[:, a // (H // G)], v[:, a // (H // G)], seen, m["scale"]) for a in range(H)]
     return torch.cat(heads, 1) @ W[p + "o"].T
 
 
@@ -127,11 +132,11 @@ def mixer_latent(h, pos, W, p: str, m: dict, eps: float) -> torch.Tensor:
     v = (c @ W[p + "uv"].T).view(T, H, dv)
     mask = m.get("mask")
     sees = (lambda i, j: sees_window(i, j, mask["size"])) if mask else (lambda i, j: j <= i)
-    heads = []
+    heads, seen = [], sight(pos, sees)
     for a in range(H):
         qa = torch.cat([q[:, a, :d], q_turned[:, a]], 1)
         ka = torch.cat([k_plain[:, a], k_turned], 1)
-        heads.append(softmax_attention(qa, ka, v[:, a], pos, m["scale"], sees))
+        heads.append(softmax_attention(qa, ka, v[:, a], seen, m["scale"]))
     o = torch.cat(heads, 1) * torch.sigmoid(h @ W[p + "g"].T)
     return o @ W[p + "o"].T
 
@@ -146,7 +151,8 @@ def mixer_chunked(h, pos, W, p: str, m: dict) -> torch.Tensor:
     mask = m.get("mask")
     sees = (lambda i, j: sees_chunk(i, j, mask["size"])) if mask else (lambda i, j: j <= i)
     gate = torch.sigmoid(h @ W[p + "g"].T)                   # [T, H]
-    heads = [softmax_attention(q[:, a], k[:, a // (H // G)], v[:, a // (H // G)], pos, m["scale"], sees) * gate[:, a:a + 1]
+    seen = sight(pos, sees)
+    heads = [softmax_attention(q[:, a], k[:, a // (H // G)], v[:, a // (H // G)], seen, m["scale"]) * gate[:, a:a + 1]
              for a in range(H)]
     return torch.cat(heads, 1) @ W[p + "o"].T
 

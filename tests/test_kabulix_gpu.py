@@ -32,7 +32,7 @@ def run_and_check(model, steps, cfg, w, reqs, dtype, what="", **kw):
     """Run the steps and hold every position against the plain implementation.  In float32 the plain run routes by
     itself.  In bfloat16 a router's close call may fall the other way and then changes every later position through
     the caches: there the plain run is told which experts the framework chose, and every such choice must be what
-    the plain router chooses once its logits may move by a fiftieth of their spread."""
+    the plain router chooses once its logits may move by a tenth of their spread."""
     if dtype == "float32":
         got, routes = run_steps(model, steps, **kw), {}
     else:
@@ -48,7 +48,7 @@ def run_and_check(model, steps, cfg, w, reqs, dtype, what="", **kw):
         for layer, taken in (forced or {}).items():
             z = seen[layer]
             for t in range(len(toks)):
-                slack = 0.02 * max(float(z[t].std()) if z.shape[1] > 1 else 1.0, 0.05)
+                slack = 0.1 * max(float(z[t].std()) if z.shape[1] > 1 else 1.0, 0.05)
                 assert P.is_close_call(z[t], taken[t], cfg["layers"][layer]["mlp"], slack), \
                     f"{what}: request {rid}, layer {layer}, position {t}: the experts {taken[t].tolist()} are not the router's choice"
         rows = got[rid]
