@@ -161,7 +161,7 @@ __device__ __forceinline__ void t32_weighted_sum(const uint4* vt, const int* vof
 // by more than T32_LAZY, so probabilities stay below 2^T32_LAZY and the accumulator is rescaled in
 // few tiles instead of most.  Sums and accumulators stay relative to the same running maximum, so
 // the result is the same.
-__device__ __forceinline__ float t32_softmax(const t32_f32x16* sc, bool edge, int p_col, int lo_col, int kb, int h,
+__device__ __forceinline__ float t32_softmax(const t32_f32x16* sc, bool edge, int p_col, int lo_col, int first, int kb, int h,
                                              float scale2, float& m_run, float& l_run, uint4* pf) {
     float sv[32];
 #pragma unroll
@@ -172,7 +172,7 @@ __device__ __forceinline__ float t32_softmax(const t32_f32x16* sc, bool edge, in
 #pragma unroll
         for (int x = 0; x < 32; ++x) {
             const int key = kb + 16 * (x >> 3) + 8 * h + (x & 7);
-            if (key > p_col || key < lo_col) sv[x] = -INFINITY;
+            if (key > p_col || (key < lo_col && key >= first)) sv[x] = -INFINITY;   // below lo only the kept first keys are seen
             asm volatile("" : "+v"(sv[x]));                  // in place and under the branch: most tiles skip all of it
         }
     }
@@ -277,6 +277,15 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
     const int khi = start + wg_last / G;
     const int klo = tl_mask_lo(mask, start + wg_col0 / G);   // of the first column: no column's is lower
     const int t_lo = klo / T32_KEYS, t_hi = khi / T32_KEYS;
+    // The tiles of the kept first keys, [0, t_head), are walked ahead of the tiles from t_lo on where the two do
+    // not touch: walk step i takes tile i below t_head and tile t_lo + i - t_head from there on.
+    int t_head = 0;
+    if (mask.first > 0 && t_lo > 0) {
+        t_head = (mask.first + T32_KEYS - 1) / T32_KEYS;
+        if (t_head > t_lo) t_head = t_lo;
+    }
+    const int t_shift = t_lo - t_head, n_tiles = t_head + t_hi - t_lo + 1;
+#define T32_TILE_AT(I) ((I) < t_head ? (I) : (I) + t_shift)
     int wk_lo = 1, wk_hi = 0, wk_full_hi = -1, wk_full_lo = 0;   // empty for a wave without columns
     if (wave_active) {
         const int w_last = ((col0 + 32 < ncols) ? col0 + 32 : ncols) - 1;
@@ -377,24 +386,25 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
 #define T32_LANDED() __builtin_amdgcn_s_waitcnt(0x0f70)
 
     __syncthreads();                                         // the page ids are in LDS
-    T32_PAGES(t_lo)
-    T32_FETCH(t_lo, 0)
-    T32_PAGES(t_lo < t_hi ? t_lo + 1 : t_hi)
+    T32_PAGES(T32_TILE_AT(0))
+    T32_FETCH(T32_TILE_AT(0), 0)
+    T32_PAGES(T32_TILE_AT(n_tiles > 1 ? 1 : 0))
     T32_LANDED();
     __syncthreads();
     int cur = 0;
-    for (int t = t_lo; t <= t_hi; ++t) {
-        if (t < t_hi) {
-            T32_FETCH(t + 1, cur ^ 1)
-            T32_PAGES(t + 2 <= t_hi ? t + 2 : t_hi)
+    for (int i = 0; i < n_tiles; ++i) {
+        const int t = T32_TILE_AT(i);
+        if (i + 1 < n_tiles) {
+            T32_FETCH(T32_TILE_AT(i + 1), cur ^ 1)
+            T32_PAGES(T32_TILE_AT(i + 2 < n_tiles ? i + 2 : n_tiles - 1))
         }
         const int kb = t * T32_KEYS;
-        if (kb <= wk_hi && kb + T32_KEYS - 1 >= wk_lo) {     // the same for the whole wave
+        if (kb <= wk_hi && (kb + T32_KEYS - 1 >= wk_lo || kb < mask.first)) {     // the same for the whole wave
             const bool edge = kb + T32_KEYS - 1 > wk_full_hi || kb < wk_full_lo;
             t32_f32x16 sc[2];
             uint4 pf[4];
             t32_scores<DC>(ks + cur * TILE, koff, qf, sc);
-            const float factor = t32_softmax(sc, edge, p_col, lo_col, kb, h, scale2, m_run, l_run, pf);
+            const float factor = t32_softmax(sc, edge, p_col, lo_col, mask.first, kb, h, scale2, m_run, l_run, pf);
             if (__any(factor != 1.0f)) {                     // some column's maximum moved
 #pragma unroll
                 for (int m = 0; m < DT; ++m)
@@ -410,6 +420,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
 #undef T32_FETCH
 #undef T32_PAGES
 #undef T32_LANDED
+#undef T32_TILE_AT
 
     if (!valid) return;
     // with a sink one is added to the denominator: a key of score 0 that has no value
@@ -447,8 +458,8 @@ extern "C" int tl_attention_tile32_columns(int waves) { return 32 * waves; }
 extern "C" int tl_attention_tile32(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                    const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
                                    void* out, int out_stride, int T, int S, int nq, int nkv, int d, int bs, int window,
-                                   float scale, int waves, int total_groups, int skip_single, int sink, int chunk,
-                                   hipStream_t stream) {
+                                   float scale, int waves, int total_groups, int skip_single, int sink, int keep_first,
+                                   int chunk, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_tile32: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_tile32: %d query heads are not a multiple of %d key/value heads", nq, nkv);
     TL_CHECK_ARG(tl_attention_tile32_takes(d, bs, NB, S, waves),
@@ -461,10 +472,9 @@ extern "C" int tl_attention_tile32(const void* q, int q_stride, const void* k_ca
                  "tl_attention_tile32: %d key/value heads or %d column groups are more than a launch takes", nkv, total_groups);
     TL_CHECK_ARG(scale > 0.f, "tl_attention_tile32: the score scale %g must be positive", (double)scale);
     TL_CHECK_ARG((uint64_t)nkv * d * 2 * 8 < (1ull << 31), "tl_attention_tile32: a cache slot of %d heads is too wide", nkv);
-    TL_CHECK_ARG(window >= 0 && chunk >= 0, "tl_attention_tile32: negative window or chunk");
+    TL_CHECK_ARG(window >= 0 && chunk >= 0 && keep_first >= 0, "tl_attention_tile32: negative window, chunk or kept first keys");
     if (T == 0 || S == 0 || total_groups == 0) return 0;
-    // windows and chunks; first keys kept in sight beyond them are left to the kernel of 16 columns per wave
-    const TlMask mask{window, chunk, 0};
+    const TlMask mask{window, chunk, keep_first};
     int bs_shift = 0;
     while ((1 << bs_shift) < bs) ++bs_shift;
     const size_t lds = t32_lds_bytes(d, NB, S);

@@ -898,7 +898,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
             ws_o, ws_ml = ws[:T * num_heads * nsplit * head_dim], ws[T * num_heads * nsplit * head_dim:]
         waves = 8 if path == "mfma-tile32" else _tile32_waves(plan.q_lens, plan.starts, num_heads) if path in (None, "mfma") else 0
-        if (waves and nt == 2 and nsplit == 1 and total128 > 0 and not keep_first      # kept first keys: the other kernel
+        if (waves and nt == 2 and nsplit == 1 and total128 > 0
                 and library().tl_attention_tile32_takes(head_dim, page, tables.shape[1], S, waves)):
             # prompt portions behind many keys, head size 64 or 128: 32 columns per wave on the 32x32
             # matrix-core instruction, work-groups of 256 columns
@@ -906,7 +906,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             total = sum(-(-n * G // cols) for n in q_lens) + pads
             _call("tl_attention_tile32", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
                   _ptr(q_start), _ptr(ctx_start), _ptr(out), o_stride, T, S, num_heads, num_kv_heads, head_dim, page,
-                  int(window), ctypes.c_float(scale), waves, total, skip_single, int(bool(sink)), chunk, _stream())
+                  int(window), ctypes.c_float(scale), waves, total, skip_single, int(bool(sink)), keep_first, chunk, _stream())
             return out
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,

@@ -644,23 +644,27 @@ def _masked_attention(q, k, v, scale, q_offset, window, keep_first, chunk):
     lies in the window (i - j < window) or among the first ``keep_first`` keys, and (with ``chunk``) in i's chunk."""
     n, nq, d = q.shape
     nkv = k.shape[1]
+    i = (q_offset + torch.arange(n)).view(n, 1)
+    j = torch.arange(k.shape[0]).view(1, -1)
+    seen = j <= i
+    if window:
+        seen &= (i - j < window) | (j < keep_first)
+    if chunk:
+        seen &= (j // chunk) == (i // chunk)
     out = torch.zeros(n, nq, d, dtype=torch.float64)
-    for a in range(n):
-        i = q_offset + a
-        js = [j for j in range(i + 1) if (not window or i - j < window or j < keep_first) and (not chunk or j // chunk == i // chunk)]
-        for h in range(nq):
-            g = h // (nq // nkv)
-            w = torch.softmax(torch.stack([(q[a, h] * k[j, g]).sum() * scale for j in js]), 0)
-            out[a, h] = sum(w[x] * v[j, g] for x, j in enumerate(js))
+    for h in range(nq):
+        g = h // (nq // nkv)
+        s = (q[:, h] @ k[:, g].T) * scale
+        out[:, h] = torch.softmax(s.masked_fill(~seen, float("-inf")), dim=1) @ v[:, g]
     return out
 
 
 MASK_PATHS = [("generic", torch.float32), ("generic", torch.bfloat16), ("mfma-direct", torch.bfloat16),
-              ("mfma-tile16", torch.bfloat16), ("mfma-tile16x2", torch.bfloat16), (None, torch.bfloat16)]
+              ("mfma-tile16", torch.bfloat16), ("mfma-tile16x2", torch.bfloat16), ("mfma-tile32", torch.bfloat16), (None, torch.bfloat16)]
 
 
 @pytest.mark.parametrize("path,dtype", MASK_PATHS)
-@pytest.mark.parametrize("window,keep_first,chunk", [(40, 6, 0), (100, 70, 0), (33, 1, 0), (64, 64, 0), (0, 0, 48), (0, 0, 64), (0, 0, 7)])
+@pytest.mark.parametrize("window,keep_first,chunk", [(44, 5, 0), (100, 70, 0), (33, 1, 0), (64, 64, 0), (0, 0, 48), (0, 0, 64), (0, 0, 7)])
 def test_attention_masks_in_prompt_portions(path, dtype, window, keep_first, chunk):
     """A window beside which the first keys stay in sight, and chunks of positions, in every kernel that takes
     prompt portions: portions that start at 0, behind cached tokens and in the middle of a window or chunk, beside
@@ -674,7 +678,7 @@ def test_attention_masks_in_prompt_portions(path, dtype, window, keep_first, chu
 @pytest.mark.parametrize("path,dtype", [("generic", torch.float32), ("generic", torch.bfloat16), ("mfma-direct", torch.bfloat16),
                                         (None, torch.bfloat16)])
 @pytest.mark.parametrize("split", [None, 64])
-@pytest.mark.parametrize("window,keep_first,chunk", [(40, 6, 0), (100, 70, 0), (200, 130, 0), (0, 0, 48), (0, 0, 128)])
+@pytest.mark.parametrize("window,keep_first,chunk", [(44, 5, 0), (100, 70, 0), (200, 130, 0), (0, 0, 48), (0, 0, 128)])
 def test_attention_masks_in_one_token_steps(path, dtype, split, window, keep_first, chunk):
     """The same masks where every sequence brings one token and the keys are split into runs: the kept first keys
     in a run of their own, in the run the window starts in, and over several runs."""
@@ -695,11 +699,21 @@ def test_attention_masks_show_a_loud_key_on_the_right_side_of_every_edge(path, d
           "window_out": lambda p: p - window, "chunk_in": lambda p: (p // chunk) * chunk,
           "chunk_out": lambda p: (p // chunk) * chunk - 1}[where]
     for lens, q_lens in (([160, 99, 300], [60, 1, 1]), ([120, 333, 64], None)):
-        if q_lens is None and path in ("mfma-tile16", "mfma-tile16x2"):
+        if q_lens is None and path in ("mfma-tile16", "mfma-tile16x2", "mfma-tile32"):
             continue
         got, want = _attention_case(dtype, 4, 2, 64, 16, lens, q_lens, window=window, seed=35, spike=True, path=path,
                                     spike_at=at, keep_first=keep_first, chunk=chunk, spike_gain=6.0)
         torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
+
+
+@pytest.mark.parametrize("path", ["mfma-tile32", "mfma-tile16", "mfma-tile16x2", "mfma-direct", "generic"])
+@pytest.mark.parametrize("window,keep_first,chunk", [(700, 100, 0), (300, 3, 0), (0, 0, 4096), (0, 0, 1000)])
+def test_attention_masks_in_a_long_portion_behind_thousands_of_keys(path, window, keep_first, chunk):
+    """1,200 tokens behind 7,800 cached ones: the kept first keys lie thousands of keys before the window, in tiles
+    of their own at the head of every work-group's walk; a chunk's edge falls inside the portion."""
+    got, want = _attention_case(torch.bfloat16, 8, 2, 64, 32, [9000], [1200], window=window, seed=5, path=path,
+                                keep_first=keep_first, chunk=chunk)
+    torch.testing.assert_close(got, want, **tol(torch.bfloat16, 3e-5, 2e-2))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
