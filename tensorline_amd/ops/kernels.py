@@ -866,7 +866,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             ctx1 = max([plan.starts[s] + 1 for s in singles if s < len(plan.starts)] + [1])
             split_len, nsplit = _key_splits(len(singles), num_kv_heads, ctx1, plan.fit_context)
             if route_singles or (route_singles is None and nsplit > 1 and _singles_get_own_launch(
-                    plan, singles, num_heads, num_kv_heads, head_dim, int(window))):
+                    plan, singles, num_heads, num_kv_heads, head_dim,
+                    (int(window) + keep_first) if window else chunk)):      # the most keys such a token reads
                 nt1 = 1 if G <= 16 or head_dim == 256 else 2      # a head size of 256: one column tile per wave (registers)
                 ws = torch.empty(len(singles) * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
                 n_o = len(singles) * num_heads * nsplit * head_dim
